@@ -1,0 +1,75 @@
+// C entry points of libshrike_hip: thin host launchers around the gfx950
+// kernels.  Every pointer is device memory unless said otherwise; `dtype` is
+// 0 for float32 and 1 for bfloat16; `stream` is a hipStream_t.  A call returns
+// 0 on success; otherwise shk_last_error() describes what was refused and
+// nothing was launched.  Shapes are checked on the host before any launch.
+#pragma once
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* shk_last_error(void);
+int shk_version(void);
+
+// out[i, :] = float(table[ids[i], :]); ids must lie in [0, vocab).
+int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int n, int hidden,
+              int vocab, void* stream);
+
+// Residual add fused with RMSNorm.  For each of n rows r (row index rows[r]
+// when `rows` is given, else r):  x = resid[row] (+ delta[row]);  if
+// write_resid the sum is stored back into resid;  out[r] = x * rsqrt(mean(x^2)
+// + eps) * weight.  resid is float32, delta and out have `dtype`, weight is
+// float32.
+int shk_add_rmsnorm(float* resid, const void* delta, const float* weight, float eps, void* out,
+                    int dtype, const int32_t* rows, int n, int hidden, int write_resid,
+                    void* stream);
+
+// out[i, j] = silu(gu[i, j]) * gu[i, inter + j] for j < inter; gu is [n, 2*inter].
+int shk_silu_mul(const void* gu, void* out, int dtype, int n, int inter, void* stream);
+
+// out[n, m] (+)= a[n, k] @ w[m, k]^T + bias[m].  a and w have in_dtype, out has
+// out_dtype, bias is float32 or null.  lda/ldo are row strides in elements.
+// With `accumulate` the product is added to what out holds (out_dtype float32
+// only).  The reduction order over k is the same for every row and column, so
+// a row's result does not depend on which other rows are in the call.
+int shk_gemm(const void* a, const void* w, const float* bias, void* out, int n, int m, int k,
+             int lda, int ldo, int in_dtype, int out_dtype, int accumulate, void* stream);
+
+// Position encoding and cache write for the n tokens of a step.  qkv is
+// [n, (heads + 2*kv_heads) * head_dim]: queries, keys, values.  Queries and
+// keys are rotated by position (pairs (i, i + rot_dim/2), angle position *
+// inv_freq[i]); queries are rewritten in place; keys and values go to their
+// page slots: page = tables[token_seq[t] * table_stride + position / page_size].
+// Pools are [num_pages, kv_heads, page_size, head_dim].  rot_dim 0 rotates
+// nothing; write_kv 0 leaves the pools alone.
+int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int head_dim,
+                      int rot_dim, const float* inv_freq, const int32_t* positions,
+                      const int32_t* token_seq, const int32_t* tables, int table_stride,
+                      void* k_pool, void* v_pool, int page_size, int num_pages, int write_kv,
+                      void* stream);
+
+// Causal attention of n query tokens over their sequences' paged caches.
+// Token t (position p, sequence s) reads keys j in (p - window, p] (all j <= p
+// when window <= 0) through tables[s].  q has row stride q_stride elements,
+// out is [n, heads * head_dim].  Softmax and accumulation are float32.
+int shk_attention(const void* q, int q_stride, void* out, int dtype, int n, int heads,
+                  int kv_heads, int head_dim, const int32_t* positions, const int32_t* token_seq,
+                  const int32_t* tables, int table_stride, int num_seqs, const void* k_pool,
+                  const void* v_pool, int page_size, int num_pages, int window, float scale,
+                  void* stream);
+
+// out[r] = lowest index of the largest value of logits[r, :vocab].
+int shk_argmax(const float* logits, int32_t* out, int rows, int vocab, int ld, void* stream);
+
+// Temperature / top-p sampling of one token per row (see sampling.hip).
+// temperature[r] == 0 takes the argmax.  uniforms[r] in [0, 1) is the draw.
+// `scratch` is float32 [rows, vocab].
+int shk_sample(const float* logits, int32_t* out, const float* temperature, const float* top_p,
+               const float* uniforms, float* scratch, int rows, int vocab, int ld, void* stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,53 @@
+"""Loads libshrike_hip.so (building it when it is absent) and declares its
+entry points for ctypes.  There is no fallback: without the library nothing
+in the product path runs."""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_void_p
+
+_LIB = None
+
+
+class KernelError(RuntimeError):
+    """A launcher refused its arguments or a launch failed."""
+
+
+_P, _I, _F = c_void_p, c_int, c_float
+
+_SIGNATURES = {
+    "shk_embed": [_P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _P],
+    "shk_silu_mul": [_P, _P, _I, _I, _I, _P],
+    "shk_gemm": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _P],
+    "shk_argmax": [_P, _P, _I, _I, _I, _P],
+    "shk_sample": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+}
+
+
+def load():
+    """The loaded library; compiles it first if no built copy matches the sources."""
+    global _LIB
+    if _LIB is None:
+        from ..csrc.build import ensure_built
+
+        path = ensure_built()
+        lib = ctypes.CDLL(str(path))
+        lib.shk_last_error.restype = c_char_p
+        lib.shk_last_error.argtypes = []
+        lib.shk_version.restype = c_int
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.argtypes = argtypes
+            fn.restype = c_int
+        lib._path = str(path)
+        _LIB = lib
+    return _LIB
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise KernelError(load().shk_last_error().decode())

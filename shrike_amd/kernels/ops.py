@@ -1,0 +1,190 @@
+"""Python faces of the HIP launchers: they take torch tensors (used purely as
+device allocations), check dtypes and contiguity, and pass raw pointers and
+the current HIP stream to libshrike_hip.  Nothing here computes anything."""
+
+from __future__ import annotations
+
+import torch
+
+from .lib import KernelError, check, load
+
+F32, BF16 = 0, 1
+_CODES = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _CODES[dtype]
+    except KeyError:
+        raise KernelError(f"kernels take float32 or bfloat16 tensors, got {dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(t: torch.Tensor, name: str, dtype=None) -> int:
+    if not t.is_cuda:
+        raise KernelError(f"{name}: expected a device tensor (there is no CPU path)")
+    if dtype is not None and t.dtype != dtype:
+        raise KernelError(f"{name}: expected {dtype}, got {t.dtype}")
+    return t.data_ptr()
+
+
+def _rows(t: torch.Tensor, name: str) -> None:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{name}: expected a 2-d tensor with unit inner stride")
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    """out[i] = float(table[ids[i]]); ids int32 [n], out float32 [n, hidden]."""
+    n, hidden = out.shape
+    if not (table.is_contiguous() and out.is_contiguous() and table.shape[1] == hidden):
+        raise KernelError("embed: table/out must be contiguous with the same width")
+    check(
+        load().shk_embed(
+            _dev(table, "table"), dtype_code(table.dtype), _dev(ids, "ids", torch.int32),
+            _dev(out, "out", torch.float32), n, hidden, table.shape[0], _stream(),
+        )
+    )
+
+
+def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_resid=True) -> None:
+    """resid (+= delta); out = rmsnorm(resid) * weight.  With `rows` (int32 [n])
+    only those rows are normed, into out[0..n)."""
+    n, hidden = out.shape
+    if not (resid.is_contiguous() and out.is_contiguous() and resid.shape[1] == hidden):
+        raise KernelError("add_rmsnorm: resid/out must be contiguous with the same width")
+    if delta is not None and (
+        delta.dtype != out.dtype or not delta.is_contiguous() or delta.shape != resid.shape
+    ):
+        raise KernelError("add_rmsnorm: delta must match resid's shape and out's dtype")
+    if weight.numel() != hidden:
+        raise KernelError(f"add_rmsnorm: weight has {weight.numel()} elements, hidden is {hidden}")
+    if rows is None and resid.shape[0] != n:
+        raise KernelError("add_rmsnorm: out and resid differ in rows")
+    check(
+        load().shk_add_rmsnorm(
+            _dev(resid, "resid", torch.float32),
+            None if delta is None else _dev(delta, "delta"),
+            _dev(weight, "weight", torch.float32), float(eps), _dev(out, "out"),
+            dtype_code(out.dtype), None if rows is None else _dev(rows, "rows", torch.int32),
+            n, hidden, int(bool(write_resid)), _stream(),
+        )
+    )
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
+    n, inter = out.shape
+    if gate_up.shape != (n, 2 * inter) or not gate_up.is_contiguous() or not out.is_contiguous():
+        raise KernelError("silu_mul: gate_up must be contiguous [n, 2*inter]")
+    if gate_up.dtype != out.dtype:
+        raise KernelError("silu_mul: dtypes differ")
+    check(load().shk_silu_mul(_dev(gate_up, "gate_up"), _dev(out, "out"), dtype_code(out.dtype),
+                              n, inter, _stream()))
+
+
+def gemm(a, w, out, bias=None, accumulate=False) -> None:
+    """out (+)= a @ w.T + bias;  a [n, k], w [m, k] contiguous, out [n, m]."""
+    _rows(a, "gemm a")
+    _rows(out, "gemm out")
+    n, k = a.shape
+    m = w.shape[0]
+    if w.dim() != 2 or w.shape[1] != k or not w.is_contiguous():
+        raise KernelError(f"gemm: w must be contiguous [m, {k}], got {tuple(w.shape)}")
+    if out.shape != (n, m):
+        raise KernelError(f"gemm: out must be [{n}, {m}], got {tuple(out.shape)}")
+    if a.dtype != w.dtype:
+        raise KernelError(f"gemm: a is {a.dtype} but w is {w.dtype}")
+    if bias is not None and bias.numel() != m:
+        raise KernelError(f"gemm: bias has {bias.numel()} elements, m is {m}")
+    check(
+        load().shk_gemm(
+            _dev(a, "a"), _dev(w, "w"),
+            None if bias is None else _dev(bias, "bias", torch.float32),
+            _dev(out, "out"), n, m, k, a.stride(0), out.stride(0),
+            dtype_code(a.dtype), dtype_code(out.dtype), int(bool(accumulate)), _stream(),
+        )
+    )
+
+
+def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, token_seq,
+                  tables, k_pool, v_pool, page_size, write_kv=True) -> None:
+    """Rotate q and k of qkv [n, (heads + 2 kv_heads) head_dim] in float32 and put
+    k, v into their pages; pools are [pages, kv_heads, page_size, head_dim]."""
+    n = qkv.shape[0]
+    if not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
+        raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim]")
+    num_pages = 0
+    if write_kv:
+        want = (k_pool.shape[0], kv_heads, page_size, head_dim)
+        if tuple(k_pool.shape) != want or tuple(v_pool.shape) != want:
+            raise KernelError(f"rope_kv_store: pools must be {want}, got {tuple(k_pool.shape)}")
+        if k_pool.dtype != qkv.dtype or v_pool.dtype != qkv.dtype:
+            raise KernelError("rope_kv_store: pools and qkv differ in dtype")
+        if not (k_pool.is_contiguous() and v_pool.is_contiguous() and tables.is_contiguous()):
+            raise KernelError("rope_kv_store: pools and tables must be contiguous")
+        num_pages = k_pool.shape[0]
+    check(
+        load().shk_rope_kv_store(
+            _dev(qkv, "qkv"), dtype_code(qkv.dtype), n, heads, kv_heads, head_dim, rot_dim,
+            None if inv_freq is None else _dev(inv_freq, "inv_freq", torch.float32),
+            _dev(positions, "positions", torch.int32),
+            _dev(token_seq, "token_seq", torch.int32) if write_kv else None,
+            _dev(tables, "tables", torch.int32) if write_kv else None,
+            tables.shape[1] if write_kv else 0,
+            _dev(k_pool, "k_pool") if write_kv else None,
+            _dev(v_pool, "v_pool") if write_kv else None,
+            page_size, num_pages, int(bool(write_kv)), _stream(),
+        )
+    )
+
+
+def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k_pool, v_pool,
+              page_size, window, scale) -> None:
+    """q: [n, >= heads*head_dim] rows (a view into qkv is fine); out [n, heads*head_dim]."""
+    _rows(q, "attention q")
+    n = q.shape[0]
+    if out.shape != (n, heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelError("attention: out must be contiguous [n, heads*head_dim] of q's dtype")
+    want = (k_pool.shape[0], kv_heads, page_size, head_dim)
+    if tuple(k_pool.shape) != want or tuple(v_pool.shape) != want:
+        raise KernelError(f"attention: pools must be {want}, got {tuple(k_pool.shape)}")
+    if k_pool.dtype != q.dtype or v_pool.dtype != q.dtype:
+        raise KernelError("attention: pools and q differ in dtype")
+    if not (k_pool.is_contiguous() and v_pool.is_contiguous() and tables.is_contiguous()):
+        raise KernelError("attention: pools and tables must be contiguous")
+    check(
+        load().shk_attention(
+            _dev(q, "q"), q.stride(0), _dev(out, "out"), dtype_code(q.dtype), n, heads, kv_heads,
+            head_dim, _dev(positions, "positions", torch.int32),
+            _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32),
+            tables.shape[1], tables.shape[0], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"),
+            page_size, k_pool.shape[0], int(window or 0), float(scale), _stream(),
+        )
+    )
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """out[r] = lowest index of the maximum of logits[r]; logits float32 [rows, vocab]."""
+    _rows(logits, "argmax logits")
+    rows, vocab = logits.shape
+    check(load().shk_argmax(_dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32),
+                            rows, vocab, logits.stride(0), _stream()))
+
+
+def sample(logits, out, temperature, top_p, uniforms, scratch) -> None:
+    """One token per row: argmax where temperature is 0, else a top-p draw with uniforms[r]."""
+    _rows(logits, "sample logits")
+    rows, vocab = logits.shape
+    if scratch.numel() < rows * vocab:
+        raise KernelError("sample: scratch needs rows * vocab float32 elements")
+    check(
+        load().shk_sample(
+            _dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32),
+            _dev(temperature, "temperature", torch.float32), _dev(top_p, "top_p", torch.float32),
+            _dev(uniforms, "uniforms", torch.float32), _dev(scratch, "scratch", torch.float32),
+            rows, vocab, logits.stride(0), _stream(),
+        )
+    )

@@ -1,0 +1,173 @@
+"""Interfaces of the parts a layer is put together from, and their registries.
+
+A part is built from its spec (``shrike_amd.config.specs``) and the model's
+width; it never sees which model it is in.  It declares the tensors it needs
+(`params`), takes them (`load`), and runs on a step's flat token batch
+(`forward`).  Kinds of parts:
+
+* Norm:              forward(ctx, hidden) -> normed [N, width] in the compute dtype;
+                     folds hidden.pending into hidden.resid first.
+* PositionEncoding:  tells a mixer how queries and keys depend on position.
+* Mixer:             forward(ctx, x, cache) -> [N, width]; mixes information
+                     between the tokens of a sequence, through `cache`
+                     (pages of keys/values, or a state slot per request).
+* FeedForward:       forward(ctx, x) -> [N, width]; token by token.
+* Block:             forward(ctx, hidden, cache) ; arranges norms, mixer and
+                     feed-forward around the residual stream.
+
+To add a part: write its spec dataclass with a unique ``kind``, write the
+class, and register it with the matching ``register_*`` function.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    """One tensor a part needs from the weight file.
+
+    init: how the random-weights mode draws it: "matrix" and "bias" are
+        N(0, 0.02), "norm" is 1 + N(0, 0.1).
+    keep_float32: held in float32 whatever the compute dtype (vectors that
+        enter float32 arithmetic); others are held in the compute dtype.
+    """
+
+    name: str
+    shape: tuple[int, ...]
+    init: str = "matrix"
+    keep_float32: bool = False
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class PagedKVSpec:
+    """Cache need of a mixer: keys and values per token, kept for all earlier
+    tokens (window None) or for the last `window` of them."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Cache need of a mixer: one tensor of fixed shape per request."""
+
+    shape: tuple[int, ...]
+    dtype: str = "float32"
+
+
+class HiddenState:
+    """The residual stream of a step: `resid` float32 [N, width], plus a part's
+    output `pending` (compute dtype) that has not been added yet.  The next
+    norm adds it while it reads the row anyway."""
+
+    __slots__ = ("resid", "pending")
+
+    def __init__(self, resid: torch.Tensor, pending: torch.Tensor | None = None):
+        self.resid = resid
+        self.pending = pending
+
+
+class Part:
+    """Common face of every part."""
+
+    def __init__(self, spec, width: int, name: str):
+        self.spec = spec
+        self.width = width
+        self.name = name
+
+    def params(self) -> list[ParamSpec]:
+        return []
+
+    def load(self, tensors: dict[str, torch.Tensor], runtime) -> None:
+        """`tensors` maps each declared name to a device tensor."""
+
+    def check(self, runtime) -> None:
+        """Raise if the kernels cannot take this part's sizes."""
+
+
+class Norm(Part):
+    def forward(self, ctx, hidden: HiddenState, rows=None, write_resid=True) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary_table(self):
+        """(inv_freq float32 [rot_dim/2], rot_dim) when the encoding is a
+        half-split rotation that the cache-write kernel applies; else None."""
+        return None
+
+    def apply(self, ctx, qkv: torch.Tensor, heads: int, kv_heads: int, head_dim: int) -> None:
+        """Encode queries and keys of qkv in place (for encodings without a fused kernel)."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        """PagedKVSpec, StateSpec or None."""
+        return None
+
+    def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block(Part):
+    mixer: Mixer
+
+    def forward(self, ctx, hidden: HiddenState, cache) -> None:
+        raise NotImplementedError
+
+
+_REGISTRIES: dict[str, dict[str, Callable]] = {
+    "norm": {},
+    "position": {},
+    "mixer": {},
+    "ffn": {},
+    "block": {},
+}
+
+
+def _register(family: str, kind: str, cls) -> None:
+    _REGISTRIES[family][kind] = cls
+
+
+def register_norm(kind: str, cls) -> None:
+    _register("norm", kind, cls)
+
+
+def register_position(kind: str, cls) -> None:
+    _register("position", kind, cls)
+
+
+def register_mixer(kind: str, cls) -> None:
+    _register("mixer", kind, cls)
+
+
+def register_ffn(kind: str, cls) -> None:
+    _register("ffn", kind, cls)
+
+
+def register_block(kind: str, cls) -> None:
+    _register("block", kind, cls)
+
+
+def build_part(family: str, spec, width: int, name: str):
+    """The part registered for ``spec.kind`` in `family`, built for `width`."""
+    kind = getattr(spec, "kind", None)
+    try:
+        cls = _REGISTRIES[family][kind]
+    except KeyError:
+        known = ", ".join(sorted(_REGISTRIES[family])) or "none"
+        raise ValueError(f"no {family} part of kind {kind!r} is registered (known: {known})") from None
+    return cls(spec, width, name)

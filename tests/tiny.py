@@ -1,0 +1,85 @@
+"""Tiny configurations of the architecture for tests.  A and B differ in every
+size and option; C has an explicit head_dim (heads * head_dim != hidden) and a
+window on its later layers."""
+
+from __future__ import annotations
+
+import json
+import tempfile
+from pathlib import Path
+
+TINY_A = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 64,
+    "intermediate_size": 172,
+    "num_hidden_layers": 2,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "vocab_size": 256,
+    "rope_theta": 10000.0,
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": True,
+    "max_position_embeddings": 128,
+    "eos_token_id": 255,
+    "torch_dtype": "float32",
+    "use_sliding_window": False,
+    "sliding_window": 32,
+}
+
+TINY_B = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "model_type": "qwen2",
+    "hidden_size": 128,
+    "intermediate_size": 352,
+    "num_hidden_layers": 3,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 1,
+    "head_dim": 32,
+    "vocab_size": 503,
+    "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-5,
+    "tie_word_embeddings": False,
+    "max_position_embeddings": 256,
+    "eos_token_id": [501, 502],
+    "torch_dtype": "float32",
+}
+
+TINY_C = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "hidden_size": 96,
+    "intermediate_size": 200,
+    "num_hidden_layers": 4,
+    "num_attention_heads": 6,
+    "num_key_value_heads": 3,
+    "head_dim": 48,
+    "vocab_size": 311,
+    "rope_theta": 50000.0,
+    "rms_norm_eps": 3e-6,
+    "tie_word_embeddings": False,
+    "torch_dtype": "float32",
+    "use_sliding_window": True,
+    "sliding_window": 24,
+    "max_window_layers": 2,
+}
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+SEEDS = {"A": 11, "B": 23, "C": 37}
+PAGE_SIZES = {"A": 4, "B": 8, "C": 16}
+
+
+def make_model_dir(name: str, root=None, dtype: str = "float32") -> Path:
+    """Writes the tiny model `name` with seeded random weights into a fresh
+    temporary folder (or `root`/name) and returns the folder."""
+    from shrike_amd.weights import write_model_folder
+
+    if root is None:
+        root = tempfile.mkdtemp(prefix="shrike_tiny_")
+    path = Path(root) / f"tiny_{name}_{dtype}"
+    if not (path / "model.safetensors").is_file():
+        write_model_folder(dict(CONFIGS[name]), path, seed=SEEDS[name], dtype=dtype)
+    return path
+
+
+def read_config(path) -> dict:
+    return json.loads((Path(path) / "config.json").read_text())
