@@ -1,0 +1,3 @@
+from .request import Request, SamplingParams, Status
+
+__all__ = ["Request", "SamplingParams", "Status"]

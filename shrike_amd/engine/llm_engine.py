@@ -1,0 +1,244 @@
+"""LLMEngine ties the step function, the scheduler and the sampler into a loop:
+step() = schedule -> one batched forward -> sample -> append / finish.
+
+Reference: shrike/engine/engine.py (same public names: add_request, has_work,
+step, generate, metrics, StepOutput).
+"""
+
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+
+import torch
+
+from ..cache import CacheManager
+from ..config.engine_config import EngineConfig
+from ..sampling import Sampler
+from .loading import load_model
+from .request import Request, SamplingParams
+from .runner import ModelRunner, StepEntry
+from .scheduler import Scheduler
+
+
+@dataclass
+class StepOutput:
+    req_id: int
+    token_id: int
+    finished: bool
+    finish_reason: str | None
+
+
+@dataclass
+class EngineStats:
+    steps: int = 0
+    tokens_generated: int = 0
+    started_at: float = field(default_factory=time.perf_counter)
+
+
+class LLMEngine:
+    """LLMEngine(model_dir, block_size=16, gpu_mem_util=0.85,
+    max_tokens_per_step=512, max_running=256, enable_prefix_caching=True,
+    num_kv_blocks=None, dtype=None, seed=0)."""
+
+    def __init__(self, model_dir: str, config: EngineConfig | None = None, *, model=None,
+                 runtime=None, **options) -> None:
+        self.config = config if config is not None else EngineConfig(**options)
+        cfg = self.config
+        self.model_dir = model_dir
+        if model is None:
+            model, runtime, _ = load_model(model_dir, cfg.dtype, cfg.device)
+        self.model, self.runtime = model, runtime
+        self.tokenizer = _load_tokenizer(model_dir) if model_dir is not None else None
+
+        specs = model.cache_specs()
+        elem = torch.empty(0, dtype=runtime.dtype).element_size()
+        probe = CacheManager(specs, cfg.block_size, 1, max_slots=1)
+        if cfg.num_kv_blocks is not None:
+            num_blocks = cfg.num_kv_blocks
+        else:
+            # shrike/engine/model_runner.py:165-174: a share of the free device memory
+            free, _total = torch.cuda.mem_get_info(runtime.device)
+            per_page = max(1, probe.bytes_per_page(elem))
+            num_blocks = max(1, int(free * cfg.gpu_mem_util) // per_page)
+        self.cache = CacheManager(specs, cfg.block_size, num_blocks, max_slots=cfg.max_running,
+                                  enable_prefix_caching=cfg.enable_prefix_caching)
+        self.cache.allocate(runtime.dtype, runtime.device)
+        self.runner = ModelRunner(model, self.cache, runtime)
+        self.scheduler = Scheduler(self.cache, cfg.max_tokens_per_step, cfg.max_running)
+        self.sampler = Sampler(runtime.device, cfg.seed)
+        self.eos_ids = set(model.spec.eos_token_ids)
+        self.requests: dict[int, Request] = {}
+        self.stats = EngineStats()
+
+    # reference name for the cache manager
+    @property
+    def block_manager(self) -> CacheManager:
+        return self.cache
+
+    def add_request(self, prompt, sampling: SamplingParams, chat: bool = True) -> int:
+        if isinstance(prompt, str):
+            token_ids = _encode(self.tokenizer, self.model_dir, prompt, chat)
+        else:
+            token_ids = [int(t) for t in prompt]
+        if not token_ids:
+            raise ValueError(
+                "empty prompt: a request must have at least one token "
+                "(the prompt tokenized to zero tokens)"
+            )
+        vocab = self.model.spec.vocab_size
+        if min(token_ids) < 0 or max(token_ids) >= vocab:
+            raise ValueError(f"prompt token ids must lie in [0, {vocab})")
+        bs = self.cache.page_size
+        worst = -(-(len(token_ids) + sampling.max_new_tokens) // bs)
+        if worst > self.cache.num_pages:
+            raise ValueError(
+                f"request needs up to {worst} KV blocks ({len(token_ids)} prompt + "
+                f"{sampling.max_new_tokens} generated tokens, block_size={bs}) but the pool has "
+                f"only {self.cache.num_pages}; it could never be scheduled - shorten the prompt, "
+                "lower max_new_tokens, or raise gpu_mem_util / num_kv_blocks"
+            )
+        req = Request(token_ids=token_ids, sampling=sampling)
+        self.requests[req.req_id] = req
+        self.scheduler.add(req)
+        return req.req_id
+
+    @property
+    def has_work(self) -> bool:
+        return self.scheduler.has_work
+
+    def step(self) -> list[StepOutput]:
+        batch = self.scheduler.schedule()
+        if not batch:
+            return []
+        entries, sampled = [], []
+        for req, n_new in batch:
+            start = req.num_computed_tokens
+            reaches_end = start + n_new >= req.num_tokens
+            entries.append(
+                StepEntry(req.cache, req.token_ids[start : start + n_new], start,
+                          [n_new - 1] if reaches_end else [])
+            )
+            if reaches_end:
+                sampled.append(req)
+        logits = self.runner.step(entries)
+        tokens = self.sampler.sample(logits, sampled)
+        for req, token in zip(sampled, tokens):
+            req.token_ids.append(token)
+
+        # before finishing: finish() gives the pages back
+        self.scheduler.postprocess(batch)
+
+        outputs: list[StepOutput] = []
+        for req, token in zip(sampled, tokens):
+            self.stats.tokens_generated += 1
+            finished, reason = False, None
+            if token in self.eos_ids and not req.sampling.ignore_eos:
+                finished, reason = True, "stop"
+            elif req.num_generated >= req.sampling.max_new_tokens:
+                finished, reason = True, "length"
+            outputs.append(StepOutput(req.req_id, token, finished, reason))
+            if finished:
+                self.scheduler.finish(req, reason)
+                del self.requests[req.req_id]
+        self.stats.steps += 1
+        return outputs
+
+    def generate(self, prompts, sampling, chat: bool = True) -> list[list[int]]:
+        """Generated token ids per prompt (the end-of-sequence token included when hit)."""
+        if isinstance(sampling, SamplingParams):
+            sampling = [sampling] * len(prompts)
+        if len(sampling) != len(prompts):
+            raise ValueError("one SamplingParams per prompt, or one for all")
+        id_map = {self.add_request(p, s, chat): i for i, (p, s) in enumerate(zip(prompts, sampling))}
+        results: list[list[int]] = [[] for _ in prompts]
+        while self.has_work:
+            for out in self.step():
+                results[id_map[out.req_id]].append(out.token_id)
+        return results
+
+    def abort(self, req_id: int) -> None:
+        req = self.requests.pop(req_id, None)
+        if req is not None:
+            self.scheduler.abort(req)
+
+    def metrics(self) -> dict:
+        sched, cache = self.scheduler, self.cache
+        elapsed = time.perf_counter() - self.stats.started_at
+        return {
+            "steps": self.stats.steps,
+            "tokens_generated": self.stats.tokens_generated,
+            "avg_tokens_per_sec": round(self.stats.tokens_generated / max(elapsed, 1e-9), 1),
+            "running": len(sched.running),
+            "waiting": len(sched.waiting),
+            "kv_blocks_total": cache.num_pages,
+            "kv_blocks_free": cache.num_free,
+            "preemptions": sched.num_preemptions,
+            "prefix_cache_hit_rate": round(
+                cache.cache_hit_blocks / max(1, cache.cache_query_blocks), 3
+            ),
+        }
+
+
+class LLM:
+    """Python entry point: LLM(model_dir, **engine options).generate(prompts, sampling_params)."""
+
+    def __init__(self, model: str, **options):
+        self.engine = LLMEngine(model, **options)
+
+    def generate(self, prompts, sampling_params: SamplingParams | list | None = None,
+                 chat: bool = False) -> list[list[int]]:
+        if sampling_params is None:
+            sampling_params = SamplingParams()
+        if prompts and isinstance(prompts[0], int):
+            prompts = [prompts]
+        return self.engine.generate(list(prompts), sampling_params, chat=chat)
+
+
+# ------------------------------------------------------------------- tokenizer
+
+
+def _load_tokenizer(model_dir):
+    """The `tokenizers` library's tokenizer from tokenizer.json, if the folder has one."""
+    import os
+
+    path = os.path.join(str(model_dir), "tokenizer.json")
+    if not os.path.isfile(path):
+        return None
+    from tokenizers import Tokenizer
+
+    return Tokenizer.from_file(path)
+
+
+def _chat_template(model_dir) -> str | None:
+    import json
+    import os
+
+    path = os.path.join(str(model_dir), "tokenizer_config.json")
+    if not os.path.isfile(path):
+        return None
+    with open(path) as f:
+        return json.load(f).get("chat_template")
+
+
+def apply_chat_template(model_dir, messages: list[dict]) -> str:
+    """Render messages with the folder's own chat template (tokenizer_config.json)."""
+    template = _chat_template(model_dir)
+    if template is None:
+        raise ValueError(f"{model_dir!r} has no chat template; pass chat=False or token ids")
+    try:
+        import jinja2
+    except ImportError:
+        raise ValueError("rendering a chat template needs jinja2; pass chat=False or token ids") from None
+    env = jinja2.Environment(trim_blocks=True, lstrip_blocks=True)
+    return env.from_string(template).render(messages=messages, add_generation_prompt=True)
+
+
+def _encode(tokenizer, model_dir, prompt: str, chat: bool) -> list[int]:
+    if tokenizer is None:
+        raise ValueError(
+            f"{model_dir!r} has no tokenizer.json: text prompts need one; pass token ids instead"
+        )
+    if chat:
+        prompt = apply_chat_template(model_dir, [{"role": "user", "content": prompt}])
+    return list(tokenizer.encode(prompt, add_special_tokens=False).ids)

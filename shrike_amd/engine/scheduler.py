@@ -1,0 +1,138 @@
+"""Continuous batching under a token budget, with chunked prompts, first-come
+first-served admission and preemption when pages run out.
+
+Behaviour follows shrike/engine/scheduler.py:69-148:
+  1. Running requests are served first, in admission order.  A request with
+     one uncomputed token costs 1; one with more (a prompt in progress, or a
+     preempted request catching up) gets a portion that fits the rest of the
+     budget.
+  2. What is left of the budget admits waiting requests, head of the queue
+     only; a prompt is cut by the budget.  If the head's portion does not fit
+     in the free pages, admission stops (nothing overtakes it, nothing is
+     preempted for it).
+  3. When a running request cannot get the pages for its portion, the newest
+     running request is preempted: all it holds goes back, it will recompute
+     from its first token, and it returns to the head of the waiting queue.
+     If the request that needs pages is itself the newest, it is the victim
+     and sits this step out.
+
+One difference: a request that resumes after preemption recomputes its prompt
+and the tokens it had generated in portions, where the reference re-decodes
+generated tokens one per step (scheduler.py:80-86); the logits are the same.
+"""
+
+from __future__ import annotations
+
+from collections import deque
+
+from ..cache.manager import CacheManager
+from .request import Request, Status
+
+
+class Scheduler:
+    def __init__(self, cache: CacheManager, max_tokens_per_step: int = 512, max_running: int = 256):
+        self.cache = cache
+        self.max_tokens_per_step = max_tokens_per_step
+        self.max_running = max_running
+        self.waiting: deque[Request] = deque()
+        self.running: list[Request] = []
+        self.num_preemptions = 0
+
+    def add(self, req: Request) -> None:
+        self.waiting.append(req)
+
+    @property
+    def has_work(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def _release(self, req: Request) -> None:
+        if req.cache is not None:
+            self.cache.free(req.cache)
+            req.cache = None
+        req.hashed_pages, req.last_hash = 0, None
+
+    def _preempt_for(self, req: Request) -> bool:
+        """Preempt the newest running request; False if that was `req` itself."""
+        victim = self.running.pop()
+        self.num_preemptions += 1
+        self._release(victim)
+        victim.num_computed_tokens = 0
+        victim.status = Status.WAITING
+        self.waiting.appendleft(victim)
+        return victim is not req
+
+    def schedule(self) -> list[tuple[Request, int]]:
+        singles: list[tuple[Request, int]] = []
+        portions: list[tuple[Request, int]] = []
+        budget = self.max_tokens_per_step
+
+        for req in list(self.running):
+            if budget == 0:
+                break
+            if req.status is not Status.RUNNING:  # preempted earlier in this step
+                continue
+            n_new = min(req.num_tokens - req.num_computed_tokens, budget)
+            if n_new <= 0:
+                continue
+            while not self.cache.can_append(req.cache, req.num_computed_tokens, n_new):
+                if not self._preempt_for(req):
+                    n_new = 0
+                    break
+            if n_new == 0:
+                continue
+            self.cache.append(req.cache, req.num_computed_tokens, n_new)
+            (singles if n_new == 1 else portions).append((req, n_new))
+            budget -= n_new
+
+        while (
+            self.waiting
+            and budget > 0
+            and len(self.running) < self.max_running
+            and self.cache.slots.num_free > 0
+        ):
+            req = self.waiting[0]
+            seq = self.cache.new_sequence()
+            # A resumed request recomputes what it generated before it was preempted too.
+            known = req.num_tokens
+            cached = self.cache.match_prefix(seq, req.token_ids[: req.num_prompt_tokens])
+            n_new = min(known - cached, budget)
+            if not self.cache.can_append(seq, cached, n_new):
+                self.cache.free(seq)  # also drops the references a prefix match took
+                break
+            self.waiting.popleft()
+            req.cache = seq
+            req.num_computed_tokens = cached
+            req.hashed_pages, req.last_hash = 0, None
+            self.cache.append(seq, cached, n_new)
+            req.status = Status.RUNNING
+            self.running.append(req)
+            (singles if n_new == 1 else portions).append((req, n_new))
+            budget -= n_new
+
+        return singles + portions
+
+    def postprocess(self, batch: list[tuple[Request, int]]) -> None:
+        """Count the step's tokens as computed, publish full pages for prefix
+        sharing, and give back pages that a window has passed."""
+        for req, n_new in batch:
+            req.num_computed_tokens += n_new
+            req.hashed_pages, req.last_hash = self.cache.register_full_pages(
+                req.cache, req.token_ids, req.num_computed_tokens, req.hashed_pages, req.last_hash
+            )
+            self.cache.trim(req.cache, req.num_computed_tokens)
+
+    def finish(self, req: Request, reason: str) -> None:
+        req.status = Status.FINISHED
+        req.finish_reason = reason
+        self.running.remove(req)
+        self._release(req)
+
+    def abort(self, req: Request) -> None:
+        """Drop a request wherever it is (command line interrupt)."""
+        if req in self.running:
+            self.finish(req, "aborted")
+            return
+        if req in self.waiting:
+            self.waiting.remove(req)
+        self._release(req)
+        req.status, req.finish_reason = Status.FINISHED, "aborted"

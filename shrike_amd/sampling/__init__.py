@@ -1,0 +1,3 @@
+from .sampler import Sampler, splitmix64, uniform
+
+__all__ = ["Sampler", "splitmix64", "uniform"]

@@ -1,0 +1,61 @@
+"""Choosing next tokens from the logits of a step: greedy, temperature, top-p,
+mixed per row, on the device.
+
+Reference: shrike/engine/sampler.py:10-31.  Rows with temperature 0 take the
+argmax of the raw logits (lowest index among equal maxima); other rows draw
+from softmax(logits / T) restricted to the top-p nucleus.  The reference draws
+with torch's global generator; here every draw is a pure function of
+(seed, number of the draw), so a generation can be repeated whatever else ran.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+
+_MASK = (1 << 64) - 1
+
+
+def splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    x = ((x ^ (x >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    x = ((x ^ (x >> 27)) * 0x94D049BB133111EB) & _MASK
+    return x ^ (x >> 31)
+
+
+def uniform(seed: int, draw: int) -> float:
+    """The draw-th number in [0, 1) of the stream `seed` (24 bits, exact in float32)."""
+    return (splitmix64(splitmix64(seed & _MASK) ^ (draw & _MASK)) >> 40) / float(1 << 24)
+
+
+class Sampler:
+    def __init__(self, device, engine_seed: int = 0):
+        self.device = device
+        self.engine_seed = engine_seed
+        self._scratch = None
+
+    def request_seed(self, req) -> int:
+        if req.sampling.seed is not None:
+            return req.sampling.seed
+        return splitmix64((self.engine_seed << 20) ^ req.req_id)
+
+    def sample(self, logits: torch.Tensor, reqs: list) -> list[int]:
+        """logits float32 [R, vocab] on the device, one row per request."""
+        if not reqs:
+            return []
+        rows, vocab = logits.shape
+        out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        if all(r.sampling.temperature == 0.0 for r in reqs):
+            ops.argmax(logits, out)
+            return out.tolist()
+        params = torch.tensor(
+            [[r.sampling.temperature for r in reqs],
+             [r.sampling.top_p for r in reqs],
+             [uniform(self.request_seed(r), r.num_generated) for r in reqs]],
+            dtype=torch.float32,
+        ).to(logits.device)
+        if self._scratch is None or self._scratch.numel() < rows * vocab:
+            self._scratch = torch.empty(rows * vocab, dtype=torch.float32, device=logits.device)
+        ops.sample(logits, out, params[0], params[1], params[2], self._scratch)
+        return out.tolist()

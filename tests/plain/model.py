@@ -235,7 +235,7 @@ def softmax_sample_reference(logits: torch.Tensor, temperature: float, top_p: fl
     logits/T, sorted descending, kept where the mass before an entry is below
     top_p (the largest is always kept).  Returns (kept token ids, weights)."""
     probs = torch.softmax(logits.double() / temperature, dim=-1)
-    sorted_probs, sorted_idx = probs.sort(-1, descending=True, stable=True)
+    sorted_probs, sorted_idx = probs.sort(dim=-1, descending=True, stable=True)
     before = sorted_probs.cumsum(-1) - sorted_probs
     keep = before < top_p
     return sorted_idx[keep], sorted_probs[keep]

@@ -1,0 +1,226 @@
+"""The engine end to end on the GPU: generation through the Python entry point
+against the plain implementation, sampling, what happens when pages run out,
+prefix sharing, long decoding, and the guards of add_request."""
+
+import random
+
+import pytest
+import torch
+
+from .plain.model import PlainModel, softmax_sample_reference
+from .tiny import CONFIGS, PAGE_SIZES, make_model_dir
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def model_root(tmp_path_factory):
+    return tmp_path_factory.mktemp("models")
+
+
+def prompts_for(name, lengths, seed=0):
+    rng = random.Random(seed)
+    vocab = CONFIGS[name]["vocab_size"]
+    eos = CONFIGS[name].get("eos_token_id", [])
+    eos = set(eos if isinstance(eos, list) else [eos])
+    return [[rng.choice([t for t in range(vocab) if t not in eos]) for _ in range(n)] for n in lengths]
+
+
+def check_against_plain(plain, prompt, generated, gap, first_logits=None):
+    """Every generated token is the plain model's argmax, unless the plain
+    model's two best logits are closer than `gap` (bfloat16 near-ties; the
+    reference's tests/test_paged.py:88-99 tests the same way)."""
+    seq = list(prompt)
+    for i, tok in enumerate(generated):
+        row = plain.logits(seq)[-1]
+        if int(row.argmax()) != tok:
+            top2 = row.topk(2).values
+            assert gap > 0 and float(top2[0] - top2[1]) < gap, (
+                f"token {i}: engine chose {tok}, plain argmax {int(row.argmax())} at a clear margin"
+            )
+        seq.append(tok)
+
+
+@pytest.mark.parametrize(
+    "name, lengths, new, budget",
+    [("A", [5, 11, 17], 8, 512), ("B", [1, 9, 30, 64], 12, 16), ("C", [3, 50, 28], 40, 24)],
+)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(name, lengths, new, budget, dtype, model_root):
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir(name, model_root, dtype=dtype, mode="unit")
+    plain = PlainModel(model_dir)
+    prompts = prompts_for(name, lengths)
+    llm = LLM(str(model_dir), dtype=dtype, block_size=PAGE_SIZES[name], num_kv_blocks=64,
+              max_tokens_per_step=budget)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
+    assert [len(o) for o in outs] == [new] * len(prompts)
+    for prompt, out in zip(prompts, outs):
+        if dtype == "float32":
+            assert out == plain.greedy(prompt, new)  # identical greedy tokens
+        else:
+            check_against_plain(plain, prompt, out, gap=0.05 * float(plain.logits(prompt).abs().max()))
+    assert llm.engine.cache.num_free == llm.engine.cache.num_pages  # tests/test_paged.py:102-103
+    assert llm.engine.cache.slots.num_free == llm.engine.cache.slots.num_slots
+
+
+def test_reference_weights_greedy_identical_in_float32(model_root):
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir("A", model_root)
+    plain = PlainModel(model_dir)
+    prompts = prompts_for("A", [5, 11, 17], seed=4)
+    llm = LLM(str(model_dir), dtype="float32", block_size=4, num_kv_blocks=32, max_tokens_per_step=3)
+    outs = llm.generate(prompts, SamplingParams(max_new_tokens=8, ignore_eos=True))
+    assert outs == [plain.greedy(p, 8) for p in prompts]
+
+
+def test_eos_stops_and_is_emitted(model_root):
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir("B", model_root, mode="unit")
+    plain = PlainModel(model_dir)
+    prompt = prompts_for("B", [12], seed=9)[0]
+    free_run = plain.greedy(prompt, 30)
+    llm = LLM(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=32)
+    llm.engine.eos_ids = {free_run[6]}  # whatever the 7th token is ends the request
+    out = llm.generate([prompt], SamplingParams(max_new_tokens=30))[0]
+    stop = free_run.index(free_run[6])
+    assert out == free_run[: stop + 1]
+    out = llm.generate([prompt], SamplingParams(max_new_tokens=10, ignore_eos=True))[0]
+    assert out == free_run[:10]
+
+
+def test_temperature_sampling_is_repeatable_and_stays_in_the_nucleus(model_root):
+    from shrike_amd import LLM, SamplingParams
+
+    model_dir = make_model_dir("B", model_root, mode="unit")
+    plain = PlainModel(model_dir)
+    prompts = prompts_for("B", [1, 9, 30, 64], seed=2)
+    llm = LLM(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64, max_tokens_per_step=16)
+    sp = SamplingParams(max_new_tokens=12, temperature=0.7, top_p=0.8, seed=1234, ignore_eos=True)
+    a = llm.generate(prompts, sp)
+    b = llm.generate(list(reversed(prompts)), sp)[::-1]  # other batch order, other request ids
+    assert a == b
+    c = llm.generate(prompts, SamplingParams(max_new_tokens=12, temperature=0.7, top_p=0.8, seed=99, ignore_eos=True))
+    assert a != c
+    greedy = llm.generate(prompts, SamplingParams(max_new_tokens=12, ignore_eos=True))
+    assert a != greedy
+    for prompt, out in zip(prompts, a):
+        seq = list(prompt)
+        for tok in out:
+            kept, weights = softmax_sample_reference(plain.logits(seq)[-1], 0.7, 0.8)
+            # the rule's kept set, give or take its last entry (float32 against float64 at the edge)
+            kept2, _ = softmax_sample_reference(plain.logits(seq)[-1], 0.7, 0.8 + 1e-4)
+            assert tok in kept.tolist() or tok in kept2.tolist()
+            seq.append(tok)
+
+
+def test_when_pages_run_out_the_newest_request_is_preempted_and_recomputes(model_root):
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+
+    model_dir = make_model_dir("A", model_root, mode="unit")
+    prompts = prompts_for("A", [9, 14, 6, 11], seed=5)
+    sp = SamplingParams(max_new_tokens=20, ignore_eos=True)
+    roomy = LLMEngine(str(model_dir), dtype="float32", block_size=4, num_kv_blocks=64)
+    want = roomy.generate(prompts, sp)
+    assert roomy.metrics()["preemptions"] == 0
+    # 12 pages of 4: all four prompts fit, their generations do not
+    tight = LLMEngine(str(model_dir), dtype="float32", block_size=4, num_kv_blocks=12,
+                      enable_prefix_caching=False)
+    got = tight.generate(prompts, sp)
+    assert tight.metrics()["preemptions"] > 0
+    assert got == want
+    assert tight.cache.num_free == 12 and not tight.has_work
+
+
+def test_prefix_sharing_changes_nothing_but_the_work(model_root):
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+
+    model_dir = make_model_dir("B", model_root, mode="unit")
+    common = prompts_for("B", [40], seed=6)[0]
+    prompts = [common + tail for tail in ([5, 6, 7], [8], [9, 10, 11, 12, 13])]
+    sp = SamplingParams(max_new_tokens=6, ignore_eos=True)
+    off = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64, enable_prefix_caching=False)
+    want = [off.generate([p], sp)[0] for p in prompts]
+    on = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64)
+    got = [on.generate([p], sp)[0] for p in prompts]
+    assert got == want
+    assert on.metrics()["prefix_cache_hit_rate"] > 0.5 and off.metrics()["prefix_cache_hit_rate"] == 0
+
+
+def test_long_decoding_and_first_tokens(model_root):
+    """300 decoded tokens across many pages, and the logits at the first
+    positions of a sequence (one key, two keys, the first page's edge)."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    for dtype, tol in (("float32", 1e-4), ("bfloat16", 3e-2)):
+        model_dir = make_model_dir("C", model_root, dtype=dtype, mode="unit")
+        plain = PlainModel(model_dir)
+        model, rt, cfg = load_model(model_dir, dtype)
+        cache = CacheManager(model.cache_specs(), 16, 32, enable_prefix_caching=False)
+        cache.allocate(rt.dtype, rt.device)
+        runner = ModelRunner(model, cache, rt)
+        ids = prompts_for("C", [320], seed=7)[0]
+        want = plain.logits(ids)
+        seq = cache.new_sequence()
+        rows = []
+        for p, tok in enumerate(ids):  # every token on the single-token path, from the very first
+            cache.append(seq, p, 1)
+            rows.append(runner.step([StepEntry(seq, [tok], p, [0])]).cpu().clone())
+            cache.trim(seq, p + 1)
+        got = torch.cat(rows).double()
+        err = (got - want).abs().amax(-1) / want.abs().max()
+        assert float(err.max()) <= tol, f"{dtype}: worst at position {int(err.argmax())}: {float(err.max()):.3e}"
+        cache.free(seq)
+        cache.check([])
+
+
+def test_add_request_guards(model_root):
+    # tests/test_review_regressions.py:90-93
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+
+    engine = LLMEngine(str(make_model_dir("A", model_root)), dtype="float32", block_size=4, num_kv_blocks=8)
+    with pytest.raises(ValueError, match="empty"):
+        engine.add_request([], SamplingParams())
+    with pytest.raises(ValueError, match="never be scheduled"):
+        engine.add_request([1, 2, 3], SamplingParams(max_new_tokens=10_000_000))
+    with pytest.raises(ValueError, match="token ids"):
+        engine.add_request([1, 2, 256], SamplingParams())
+    with pytest.raises(ValueError, match="tokenizer"):
+        engine.add_request("some text", SamplingParams())
+    assert engine.step() == [] and not engine.has_work
+
+
+def test_metrics_and_streaming_outputs(model_root):
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+
+    engine = LLMEngine(str(make_model_dir("A", model_root)), dtype="bfloat16", block_size=4, num_kv_blocks=32)
+    rid = engine.add_request([1, 2, 3, 4, 5], SamplingParams(max_new_tokens=3, ignore_eos=True))
+    outs = []
+    while engine.has_work:
+        outs += engine.step()
+    assert [o.req_id for o in outs] == [rid] * 3
+    assert [o.finished for o in outs] == [False, False, True] and outs[-1].finish_reason == "length"
+    m = engine.metrics()
+    assert m["tokens_generated"] == 3 and m["steps"] == 3 and m["running"] == 0
+    assert m["kv_blocks_total"] == 32 and m["kv_blocks_free"] == 32
+
+
+def test_command_line_generates(model_root, capsys):
+    from shrike_amd.__main__ import main
+
+    model_dir = make_model_dir("A", model_root, mode="unit")
+    rc = main(["--model", str(model_dir), "--prompt-ids", "5,6,7,8", "--max-tokens", "5",
+               "--dtype", "fp32", "--block-size", "4", "--num-kv-blocks", "16", "--ignore-eos", "--metrics"])
+    assert rc == 0
+    out = capsys.readouterr()
+    assert [int(t) for t in out.out.split()] == PlainModel(model_dir).greedy([5, 6, 7, 8], 5)
+    assert "tokens_generated" in out.err

@@ -1,0 +1,362 @@
+"""Each HIP kernel alone against a plain float32/float64 torch computation of
+the same operation, at sizes the engine's tiny models do not use."""
+
+import math
+
+import pytest
+import torch
+
+from .plain import model as plain
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+TOL = {torch.float32: 5e-6, torch.bfloat16: 1e-2}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from shrike_amd.kernels import ops
+
+    return ops
+
+
+def dev(t, dtype=None):
+    return t.to("cuda", dtype) if dtype else t.to("cuda")
+
+
+def close(got, want, dtype, scale=None):
+    want = want.double().cpu()
+    scale = want.abs().max().clamp_min(1e-30) if scale is None else scale
+    err = ((got.double().cpu() - want).abs().max() / scale).item()
+    assert err <= TOL[dtype], f"rel err {err:.3e} > {TOL[dtype]}"
+
+
+def rounded(t, dtype):
+    """The values a tensor has after it is stored in `dtype`."""
+    return t.to(dtype).double()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden, vocab", [(72, 101), (3584, 777)])
+def test_embed(ops, dtype, hidden, vocab):
+    torch.manual_seed(1)
+    table = torch.randn(vocab, hidden)
+    ids = torch.randint(0, vocab, (13,), dtype=torch.int32)
+    out = torch.empty(13, hidden, device="cuda")
+    ops.embed(dev(table, dtype), dev(ids), out)
+    assert torch.equal(out.cpu(), table.to(dtype).float()[ids.long()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("hidden, eps", [(72, 1e-6), (1000, 1e-5), (5120, 3e-3)])
+def test_add_rmsnorm(ops, dtype, hidden, eps):
+    torch.manual_seed(2)
+    n = 9
+    resid, delta, w = torch.randn(n, hidden) * 3, torch.randn(n, hidden), 1 + 0.1 * torch.randn(hidden)
+    r = dev(resid.clone())
+    out = torch.empty(n, hidden, device="cuda", dtype=dtype)
+    ops.add_rmsnorm(r, dev(delta, dtype), dev(w), eps, out)
+    summed = resid.double() + rounded(delta, dtype)
+    close(r, summed, torch.float32)  # the residual sum stays float32 in both modes
+    close(out, plain.rms_norm(summed, w.double(), eps), dtype)
+    # without delta, on chosen rows, without touching the residual
+    rows = torch.tensor([4, 0, 7], dtype=torch.int32)
+    before = r.clone()
+    out2 = torch.empty(3, hidden, device="cuda", dtype=dtype)
+    ops.add_rmsnorm(r, dev(delta, dtype), dev(w), eps, out2, rows=dev(rows), write_resid=False)
+    assert torch.equal(r, before)
+    x = before.double().cpu()[rows.long()] + rounded(delta, dtype)[rows.long()]
+    close(out2, plain.rms_norm(x, w.double(), eps), dtype)
+    # a norm in the wrong place (mean subtracted, eps outside the root) fails this
+    const = torch.full((1, hidden), 2.0, device="cuda")
+    out3 = torch.empty(1, hidden, device="cuda", dtype=dtype)
+    ops.add_rmsnorm(const, None, torch.ones(hidden, device="cuda"), eps, out3)
+    close(out3, torch.full((1, hidden), 2.0 / math.sqrt(4.0 + eps)), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n, inter", [(1, 172), (7, 18944), (33, 100)])
+def test_silu_mul(ops, dtype, n, inter):
+    torch.manual_seed(3)
+    gu = torch.randn(n, 2 * inter) * 4
+    out = torch.empty(n, inter, device="cuda", dtype=dtype)
+    ops.silu_mul(dev(gu, dtype), out)
+    g, u = rounded(gu, dtype)[:, :inter], rounded(gu, dtype)[:, inter:]
+    close(out, g * torch.sigmoid(g) * u, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n, m, k", [(1, 503, 128), (5, 64, 172), (70, 130, 96), (130, 200, 333), (64, 3584, 512)])
+def test_gemm(ops, dtype, n, m, k):
+    torch.manual_seed(4)
+    a, w, b = torch.randn(n, k), torch.randn(m, k) / math.sqrt(k), torch.randn(m)
+    want = rounded(a, dtype) @ rounded(w, dtype).t() + b.double()
+    out = torch.empty(n, m, device="cuda", dtype=dtype)
+    ops.gemm(dev(a, dtype), dev(w, dtype), out, bias=dev(b))
+    close(out, want, dtype)
+    # float32 output from bfloat16 inputs (logits), without bias, accumulated on top
+    out32 = torch.ones(n, m, device="cuda")
+    ops.gemm(dev(a, dtype), dev(w, dtype), out32, accumulate=True)
+    close(out32, want - b.double() + 1.0, torch.float32 if dtype == torch.float32 else dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_gemm_rows_do_not_depend_on_the_rest_of_the_batch(ops, dtype):
+    torch.manual_seed(5)
+    a, w = dev(torch.randn(77, 200), dtype), dev(torch.randn(150, 200), dtype)
+    full = torch.empty(77, 150, device="cuda", dtype=torch.float32)
+    ops.gemm(a, w, full)
+    one = torch.empty(1, 150, device="cuda", dtype=torch.float32)
+    ops.gemm(a[40:41], w, one)
+    assert torch.equal(one[0], full[40])
+
+
+def test_gemm_refuses_what_it_cannot_do(ops):
+    from shrike_amd.kernels import KernelError
+
+    a, w = torch.zeros(2, 8, device="cuda"), torch.zeros(4, 9, device="cuda")
+    with pytest.raises(KernelError):
+        ops.gemm(a, w, torch.zeros(2, 4, device="cuda"))
+    with pytest.raises(KernelError, match="device"):
+        ops.gemm(torch.zeros(2, 8), torch.zeros(4, 8), torch.zeros(2, 4))
+    with pytest.raises(KernelError):
+        ops.gemm(a, torch.zeros(4, 8, device="cuda", dtype=torch.bfloat16), torch.zeros(2, 4, device="cuda"))
+
+
+# ------------------------------------------------------------ rotation + cache
+
+
+def paged_setup(seq_lens, page_size, num_pages, kv_heads, head_dim, dtype, seed=0):
+    """Random distinct pages per sequence; tables padded with 0 as the runner builds them."""
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(num_pages, generator=g).tolist()
+    tables, width = [], max(-(-n // page_size) for n in seq_lens)
+    for n in seq_lens:
+        need = -(-n // page_size)
+        tables.append([perm.pop() for _ in range(need)] + [0] * (width - need))
+    k_pool = torch.full((num_pages, kv_heads, page_size, head_dim), float("nan"), dtype=dtype, device="cuda")
+    v_pool = torch.full_like(k_pool, float("nan"))
+    return torch.tensor(tables, dtype=torch.int32, device="cuda"), k_pool, v_pool
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads, kv_heads, head_dim, page_size, theta", [(6, 3, 48, 8, 5e4), (14, 2, 64, 16, 1e6), (5, 5, 80, 4, 1e4)])
+def test_rope_kv_store(ops, dtype, heads, kv_heads, head_dim, page_size, theta):
+    torch.manual_seed(6)
+    seq_lens = [37, 1, 12]
+    starts = [5, 0, 3000]  # positions far out: angles of thousands of radians
+    n = sum(seq_lens)
+    tables, k_pool, v_pool = paged_setup([s + l for s, l in zip(starts, seq_lens)], page_size, 1024, kv_heads, head_dim, dtype)
+    token_seq = torch.cat([torch.full((l,), i) for i, l in enumerate(seq_lens)]).int()
+    positions = torch.cat([torch.arange(s, s + l) for s, l in zip(starts, seq_lens)]).int()
+    qkv = torch.randn(n, (heads + 2 * kv_heads) * head_dim)
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2).float() / head_dim))
+    buf = dev(qkv, dtype)
+    ops.rope_kv_store(buf, heads, kv_heads, head_dim, head_dim, dev(inv_freq), dev(positions), dev(token_seq), tables, k_pool, v_pool, page_size)
+
+    x = rounded(qkv, dtype)
+    q = x[:, : heads * head_dim].view(n, heads, head_dim)
+    k = x[:, heads * head_dim : (heads + kv_heads) * head_dim].view(n, kv_heads, head_dim)
+    v = x[:, (heads + kv_heads) * head_dim :].view(n, kv_heads, head_dim)
+    cos, sin = plain.rope_tables(positions.long(), head_dim, theta)
+    close(buf[:, : heads * head_dim].reshape(n, heads, head_dim), plain.apply_rope(q, cos, sin), dtype)
+    for t in range(n):
+        s, p = int(token_seq[t]), int(positions[t])
+        page = int(tables[s, p // page_size])
+        close(k_pool[page, :, p % page_size], plain.apply_rope(k[t : t + 1], cos[t : t + 1], sin[t : t + 1])[0], dtype)
+        assert torch.equal(v_pool[page, :, p % page_size].cpu().double(), v[t])
+    # nothing else was written: every other slot is still NaN
+    written = sum(seq_lens) * kv_heads * head_dim
+    assert int((~torch.isnan(k_pool.float())).sum()) == written
+    assert int((~torch.isnan(v_pool.float())).sum()) == written
+
+
+def reference_attention(q, k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale):
+    """Gathers each sequence's keys through its table and runs the plain attention."""
+    outs = []
+    heads = q.shape[1]
+    off = 0
+    for s, (start, n_new) in enumerate(zip(starts, seq_lens)):
+        ctx = start + n_new
+        pages = tables[s, : -(-ctx // page_size)].long().cpu()
+        k = k_pool.cpu().double()[pages].permute(0, 2, 1, 3).reshape(-1, k_pool.shape[1], k_pool.shape[3])[:ctx]
+        v = v_pool.cpu().double()[pages].permute(0, 2, 1, 3).reshape(-1, v_pool.shape[1], v_pool.shape[3])[:ctx]
+        k, v = torch.nan_to_num(k), torch.nan_to_num(v)  # slots outside the window may be poisoned
+        full_q = torch.zeros(ctx, heads, q.shape[2], dtype=torch.float64)
+        full_q[start:] = q[off : off + n_new]
+        d = q.shape[2]
+        o = plain.causal_attention(full_q * (scale / d**-0.5), k, v, window)[start:]
+        outs.append(o)
+        off += n_new
+    return torch.cat(outs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize(
+    "heads, kv_heads, head_dim, page_size, window",
+    [(14, 2, 64, 16, None), (4, 4, 16, 4, None), (28, 4, 128, 16, None), (6, 3, 48, 8, 20), (5, 1, 80, 64, None), (2, 1, 256, 16, 100)],
+)
+def test_attention_mixed_batch(ops, dtype, heads, kv_heads, head_dim, page_size, window):
+    """Portions with earlier context beside single tokens, context lengths of the
+    reference's own decode test (1, 15, 16, 17, 100, 333, 512, 7)."""
+    torch.manual_seed(7)
+    ctx = [1, 15, 16, 17, 100, 333, 512, 7, 260, 90]
+    seq_lens = [1, 1, 1, 1, 1, 1, 1, 1, 200, 90]  # two portions: 200 tokens after 60, 90 from the start
+    starts = [c - l for c, l in zip(ctx, seq_lens)]
+    num_pages = 2 * sum(-(-c // page_size) for c in ctx) + 3
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, num_pages, kv_heads, head_dim, dtype, seed=1)
+    for s, c in enumerate(ctx):  # fill each sequence's slots; everything else stays NaN
+        for p in range(c):
+            page = int(tables[s, p // page_size])
+            k_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
+            v_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
+    n = sum(seq_lens)
+    q = torch.randn(n, heads, head_dim).to(dtype)
+    token_seq = torch.cat([torch.full((l,), i) for i, l in enumerate(seq_lens)]).int()
+    positions = torch.cat([torch.arange(s, s + l) for s, l in zip(starts, seq_lens)]).int()
+    out = torch.empty(n, heads * head_dim, device="cuda", dtype=dtype)
+    scale = 0.7 * head_dim**-0.5  # not the default: the scale is a parameter
+    ops.attention(dev(q).view(n, -1), out, heads, kv_heads, head_dim, dev(positions), dev(token_seq), tables, k_pool, v_pool, page_size, window, scale)
+    want = reference_attention(q.double(), k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale)
+    assert not torch.isnan(out.float()).any(), "a slot outside the context was read"
+    close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
+    """One key far back is made to stand out; the output must be its value."""
+    torch.manual_seed(8)
+    heads, kv_heads, head_dim, page_size, ctx = 4, 2, 64, 16, 700
+    tables, k_pool, v_pool = paged_setup([ctx], page_size, 64, kv_heads, head_dim, dtype)
+    k = torch.randn(ctx, kv_heads, head_dim) * 0.1
+    v = torch.randn(ctx, kv_heads, head_dim)
+    q = torch.randn(1, heads, head_dim)
+    far = 37  # third page, far from the query at position 699
+    k[far] = q[0, ::2] * 4.0  # heads 0 and 2 are the first of each group
+    for p in range(ctx):
+        page = int(tables[0, p // page_size])
+        k_pool[page, :, p % page_size] = k[p].to(dtype)
+        v_pool[page, :, p % page_size] = v[p].to(dtype)
+    out = torch.empty(1, heads * head_dim, device="cuda", dtype=dtype)
+    ops.attention(dev(q, dtype).view(1, -1), out, heads, kv_heads, head_dim, torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"),
+                  torch.zeros(1, dtype=torch.int32, device="cuda"), tables, k_pool, v_pool, page_size, None, 1.0)
+    got = out.view(heads, head_dim).float().cpu()
+    for h in (0, 2):
+        assert torch.allclose(got[h], v[far, h // 2].to(dtype).float(), atol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_window_edge(ops, dtype):
+    """The key just outside the window would dominate if it were read."""
+    heads = kv_heads = 1
+    head_dim, page_size, ctx, window = 32, 8, 100, 24
+    tables, k_pool, v_pool = paged_setup([ctx], page_size, 32, kv_heads, head_dim, dtype)
+    torch.manual_seed(9)
+    q = torch.randn(1, 1, head_dim)
+    k = torch.randn(ctx, 1, head_dim) * 0.1
+    v = torch.randn(ctx, 1, head_dim)
+    edge = ctx - 1 - window  # first key outside
+    k[edge] = q[0] * 8.0
+    k[edge + 1] = q[0] * 0.5
+    for p in range(ctx):
+        page = int(tables[0, p // page_size])
+        k_pool[page, :, p % page_size] = k[p].to(dtype)
+        v_pool[page, :, p % page_size] = v[p].to(dtype)
+    args = (heads, kv_heads, head_dim, torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"),
+            torch.zeros(1, dtype=torch.int32, device="cuda"), tables, k_pool, v_pool, page_size)
+    out = torch.empty(1, head_dim, device="cuda", dtype=dtype)
+    ops.attention(dev(q, dtype).view(1, -1), out, *args, window, 1.0)
+    kk, vv = rounded(k, dtype), rounded(v, dtype)
+    want = plain.causal_attention(rounded(q, dtype).expand(ctx, 1, head_dim) * head_dim**0.5, kk, vv, window)[-1]
+    close(out.view(1, head_dim), want, dtype, scale=1.0)
+    out_full = torch.empty_like(out)
+    ops.attention(dev(q, dtype).view(1, -1), out_full, *args, None, 1.0)
+    assert torch.allclose(out_full.float().cpu()[0], v[edge, 0].to(dtype).float(), atol=2e-2)  # without a window the edge key wins
+
+
+def test_attention_refuses_head_sizes_it_cannot_do(ops):
+    from shrike_amd.kernels import KernelError
+
+    with pytest.raises(KernelError, match="head_dim"):
+        z = torch.zeros(1, 272, device="cuda")
+        pool = torch.zeros(2, 1, 4, 272, device="cuda")
+        i = torch.zeros(1, dtype=torch.int32, device="cuda")
+        ops.attention(z, torch.empty_like(z), 1, 1, 272, i, i, i.view(1, 1), pool, pool, 4, None, 1.0)
+
+
+# ------------------------------------------------------------------- sampling
+
+
+def test_argmax_takes_the_lowest_index_among_equal_maxima(ops):
+    torch.manual_seed(10)
+    logits = torch.randn(6, 152064)
+    logits[0, [5, 99999, 150000]] = 50.0
+    logits[1, 152063] = 60.0
+    logits[2, 0] = 60.0
+    out = torch.empty(6, dtype=torch.int32, device="cuda")
+    ops.argmax(dev(logits), out)
+    assert out.tolist() == logits.argmax(-1).tolist()
+    assert out.tolist()[:3] == [5, 152063, 0]
+    # the reference's vectors (tests/test_sampler.py:20-23)
+    small = torch.tensor([[0.1, 5.0, 0.2], [9.0, 0.0, 0.0]], device="cuda")
+    out2 = torch.empty(2, dtype=torch.int32, device="cuda")
+    ops.argmax(small, out2)
+    assert out2.tolist() == [1, 0]
+
+
+def run_sample(ops, logits, temperature, top_p, u):
+    rows, vocab = logits.shape
+    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    f = lambda x: torch.tensor(x, dtype=torch.float32, device="cuda")  # noqa: E731
+    ops.sample(dev(logits), out, f(temperature), f(top_p), f(u), torch.empty(rows * vocab, device="cuda"))
+    return out.tolist()
+
+
+def test_sample_vectors_of_the_reference(ops):
+    # tests/test_sampler.py:36-42: a dominant entry and top_p 0.5 -> always that entry
+    logits = torch.tensor([[100.0, 0.0, 0.0, 0.0]] * 8)
+    us = [0.0, 0.1, 0.3, 0.5, 0.7, 0.9, 0.999, 0.25]
+    assert run_sample(ops, logits, [1.0] * 8, [0.5] * 8, us) == [0] * 8
+    # :45-51: a greedy row beside a sampled one
+    mixed = torch.tensor([[0.0, 0.0, 7.0], [50.0, 0.0, 0.0]])
+    assert run_sample(ops, mixed, [0.0, 1.0], [1.0, 0.9], [0.5, 0.5]) == [2, 0]
+
+
+def test_sample_draws_from_the_kept_weights_in_index_order(ops):
+    """The kept set and its weights are the plain rule's; the draw is the
+    inverse of the cumulative kept weight in index order."""
+    torch.manual_seed(11)
+    vocab = 1000
+    logits = torch.randn(1, vocab) * 3
+    for temperature, top_p in [(1.0, 1.0), (0.7, 0.9), (1.5, 0.3), (0.2, 0.05)]:
+        kept, weights = plain.softmax_sample_reference(logits[0], temperature, top_p)
+        order = kept.argsort()
+        ids, w = kept[order], weights[order]
+        cum = (w / w.sum()).cumsum(0)
+        us = [i / 64 + 1 / 256 for i in range(64)]
+        got = run_sample(ops, logits.expand(64, vocab).contiguous(), [temperature] * 64, [top_p] * 64, us)
+        for u, tok in zip(us, got):
+            assert tok in ids.tolist(), f"T={temperature} top_p={top_p}: token {tok} is outside the nucleus"
+            j = int(torch.searchsorted(cum, torch.tensor(u, dtype=torch.float64), right=True))
+            near = {int(ids[min(max(j + d, 0), len(ids) - 1)]) for d in (-1, 0, 1)}  # float32 cumulative sums
+            assert tok in near
+
+
+def test_sample_keeps_as_many_equal_weights_as_the_rule_admits(ops):
+    logits = torch.zeros(1, 10)  # ten equal weights of 0.1: top_p 0.35 keeps four
+    got = set()
+    for u in [i / 40 for i in range(40)]:
+        got.update(run_sample(ops, logits, [1.0], [0.35], [u]))
+    assert got == {0, 1, 2, 3}
+
+
+def test_sample_frequencies_follow_the_distribution(ops):
+    probs = torch.tensor([0.5, 0.25, 0.125, 0.125])
+    logits = probs.log()[None].expand(4096, 4).contiguous()
+    from shrike_amd.sampling import uniform
+
+    us = [uniform(123, i) for i in range(4096)]
+    got = torch.tensor(run_sample(ops, logits, [1.0] * 4096, [1.0] * 4096, us))
+    freq = torch.bincount(got, minlength=4).float() / 4096
+    assert torch.allclose(freq, probs, atol=0.03)

@@ -1,0 +1,295 @@
+"""Each part alone against the plain functions, a layer schedule that runs a
+block twice and lets a layer read another layer's cache, and a toy mixer with
+state of its own that is registered, built and stepped from here without any
+change to the framework's files."""
+
+from dataclasses import dataclass, replace
+from typing import ClassVar
+
+import pytest
+import torch
+
+from .plain import model as plain
+
+pytestmark = pytest.mark.gpu
+
+
+def make_runner(spec, tensors_cpu, dtype=torch.float32, page_size=8, num_pages=32):
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.runner import ModelRunner
+    from shrike_amd.engine.runtime import Runtime
+    from shrike_amd.models import DecoderModel
+
+    rt = Runtime("cuda:0", dtype)
+    model = DecoderModel(spec)
+    held = {}
+    for p in model.params():
+        if p.name in tensors_cpu:
+            held[p.name] = tensors_cpu[p.name].to("cuda", torch.float32 if p.keep_float32 else dtype)
+    model.load(held, rt)
+    cache = CacheManager(model.cache_specs(), page_size, num_pages, max_slots=8, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    return ModelRunner(model, cache, rt), model, cache
+
+
+def small_spec(**changes):
+    from shrike_amd.config import AttentionSpec, BlockSpec, ModelSpec, RMSNormSpec, RotarySpec, SwiGLUSpec
+
+    norm = RMSNormSpec(eps=1e-5)
+    mixer = AttentionSpec(num_heads=4, num_kv_heads=2, head_dim=16, qkv_bias=True, out_bias=False,
+                          scale=16**-0.5, position=RotarySpec(theta=1e4, rotary_dim=16))
+    blocks = tuple(
+        BlockSpec(name=f"model.layers.{i}", mixer=mixer, ffn=SwiGLUSpec(intermediate_size=88),
+                  mixer_norm=norm, ffn_norm=norm) for i in range(2)
+    )
+    spec = ModelSpec(architecture="toy", hidden_size=48, vocab_size=97, blocks=blocks, final_norm=norm,
+                     tie_word_embeddings=False)
+    return replace(spec, **changes)
+
+
+def cpu_weights(spec, seed=0):
+    from shrike_amd.models import DecoderModel
+    from shrike_amd.weights import random_tensors
+
+    return random_tensors(DecoderModel(spec).params(), seed, torch.float32, "cpu", mode="unit")
+
+
+def step_whole(runner, cache, ids, cuts=None):
+    from shrike_amd.engine.runner import StepEntry
+
+    seq = cache.new_sequence()
+    rows, p = [], 0
+    for n in cuts or [len(ids)]:
+        cache.append(seq, p, n)
+        rows.append(runner.step([StepEntry(seq, ids[p : p + n], p, list(range(n)))]).cpu().clone())
+        p += n
+    cache.free(seq)
+    return torch.cat(rows).double()
+
+
+# ------------------------------------------------------------ parts on their own
+
+
+def part_context(n_tokens, dtype=torch.float32):
+    """A step context for parts that only need buffers."""
+    from shrike_amd.engine.context import StepContext, Workspace
+
+    dev = torch.device("cuda:0")
+    z = torch.zeros(1, dtype=torch.int32, device=dev)
+    return StepContext(dtype=dtype, device=dev, workspace=Workspace(dev), num_tokens=n_tokens, num_seqs=1,
+                       num_decode=0, token_ids=z, positions=z, token_seq=z, cu_q=z, ctx_lens=z,
+                       state_slots=z, fresh=z, out_rows=z, block_tables=[])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from shrike_amd.config import RMSNormSpec
+    from shrike_amd.engine.runtime import Runtime
+    from shrike_amd.parts import HiddenState, build_part
+
+    torch.manual_seed(0)
+    part = build_part("norm", RMSNormSpec(eps=2e-4), 200, "n")
+    assert [(p.name, p.shape, p.keep_float32) for p in part.params()] == [("n.weight", (200,), True)]
+    w = 1 + 0.1 * torch.randn(200)
+    part.load({"n.weight": w.cuda()}, Runtime("cuda:0", dtype))
+    resid, pending = torch.randn(6, 200), torch.randn(6, 200)
+    hidden = HiddenState(resid.cuda(), pending.cuda().to(dtype))
+    out = part.forward(part_context(6, dtype), hidden)
+    total = resid.double() + pending.to(dtype).double()
+    assert hidden.pending is None and torch.allclose(hidden.resid.cpu().double(), total, atol=1e-6)
+    want = plain.rms_norm(total, w.double(), 2e-4)
+    assert (out.cpu().double() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 3e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part(dtype):
+    from shrike_amd.config import SwiGLUSpec
+    from shrike_amd.engine.runtime import Runtime
+    from shrike_amd.parts import build_part
+
+    torch.manual_seed(1)
+    part = build_part("ffn", SwiGLUSpec(intermediate_size=100), 72, "mlp")
+    assert [p.shape for p in part.params()] == [(100, 72), (100, 72), (72, 100)]
+    w = {p.name: (torch.randn(p.shape) / p.shape[1] ** 0.5).to(dtype) for p in part.params()}
+    part.load({k: v.cuda() for k, v in w.items()}, Runtime("cuda:0", dtype))
+    x = torch.randn(5, 72).to(dtype)
+    out = part.forward(part_context(5, dtype), x.cuda())
+    want = plain.swiglu(x.double(), w["mlp.gate_proj.weight"].double(), w["mlp.up_proj.weight"].double(),
+                        w["mlp.down_proj.weight"].double())
+    assert (out.cpu().double() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 3e-2) * want.abs().max()
+
+
+def test_position_part_gives_the_reference_frequencies():
+    from shrike_amd.config import RotarySpec
+    from shrike_amd.engine.runtime import Runtime
+    from shrike_amd.parts import build_part
+
+    part = build_part("position", RotarySpec(theta=1e6, rotary_dim=32), 64, "rope")
+    part.load({}, Runtime("cuda:0", torch.float32))
+    inv_freq, rot_dim = part.rotary_table()
+    want = 1.0 / (1e6 ** (torch.arange(0, 32, 2).float() / 32))
+    assert rot_dim == 32 and torch.equal(inv_freq.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_part_and_block(dtype):
+    """One block alone: the mixer's declared tensors, its cache need, and its
+    output against the plain attention block and decoder layer."""
+    spec = small_spec()
+    spec = replace(spec, blocks=spec.blocks[:1], schedule=())
+    w = cpu_weights(spec, seed=3)
+    if dtype == torch.bfloat16:
+        w = {k: v.to(dtype).float() for k, v in w.items()}
+    runner, model, cache = make_runner(spec, w, dtype)
+    mixer = model.blocks[0].mixer
+    names = sorted(p.name.split("self_attn.")[1] for p in mixer.params())
+    assert names == ["k_proj.bias", "k_proj.weight", "o_proj.weight", "q_proj.bias", "q_proj.weight",
+                     "v_proj.bias", "v_proj.weight"]
+    from shrike_amd.parts import PagedKVSpec
+
+    assert mixer.cache_spec() == PagedKVSpec(2, 16, None)
+    ids = torch.randint(0, 97, (21,), generator=torch.Generator().manual_seed(1)).tolist()
+    got = step_whole(runner, cache, ids, cuts=[9, 1, 11])
+    cfg = plain.PlainConfig(48, 88, 1, 4, 2, 16, 97, 1e-5, 1e4, False)
+    want = plain.forward(cfg, {k: v.double() for k, v in w.items()}, ids)
+    assert plain.rel_err(got, want) <= (1e-5 if dtype == torch.float32 else 3e-2)
+
+
+# ------------------------------------------------------------- the order is data
+
+
+def plain_scheduled(spec, w, ids, order, cache_of):
+    """The plain model with the layers run in `order`; cache_of[i] = j makes run i
+    attend over the keys and values that run j computed."""
+    cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
+    w = {k: v.double() for k, v in w.items()}
+    n = len(ids)
+    cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+    x = w["model.embed_tokens.weight"][torch.tensor(ids)]
+    kv = {}
+    for run, layer in enumerate(order):
+        p = f"model.layers.{layer}"
+        h = plain.rms_norm(x, w[f"{p}.input_layernorm.weight"], 1e-5)
+        a = f"{p}.self_attn"
+        q = plain.apply_rope(plain.linear(h, w[f"{a}.q_proj.weight"], w[f"{a}.q_proj.bias"]).view(n, 4, 16), cos, sin)
+        if cache_of[run] is None:
+            k = plain.apply_rope(plain.linear(h, w[f"{a}.k_proj.weight"], w[f"{a}.k_proj.bias"]).view(n, 2, 16), cos, sin)
+            v = plain.linear(h, w[f"{a}.v_proj.weight"], w[f"{a}.v_proj.bias"]).view(n, 2, 16)
+            kv[run] = (k, v)
+        else:
+            k, v = kv[cache_of[run]]
+        o = plain.causal_attention(q, k, v)
+        x = x + plain.linear(o.reshape(n, -1), w[f"{a}.o_proj.weight"])
+        h = plain.rms_norm(x, w[f"{p}.post_attention_layernorm.weight"], 1e-5)
+        x = x + plain.swiglu(h, w[f"{p}.mlp.gate_proj.weight"], w[f"{p}.mlp.up_proj.weight"], w[f"{p}.mlp.down_proj.weight"])
+    x = plain.rms_norm(x, w["model.norm.weight"], 1e-5)
+    return plain.linear(x, w["lm_head.weight"])
+
+
+def test_schedule_may_name_a_layer_twice_and_share_a_cache():
+    from shrike_amd.config import ScheduleEntry
+
+    schedule = (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_of=1))
+    spec = small_spec(schedule=schedule)
+    w = cpu_weights(spec, seed=4)
+    runner, model, cache = make_runner(spec, w)
+    assert [c is not None for c in model.cache_specs()] == [True, True, True, False]
+    assert len(cache.groups) == 1 and cache.groups[0].layers == [0, 1, 2]
+    ids = torch.randint(0, 97, (30,), generator=torch.Generator().manual_seed(2)).tolist()
+    want = plain_scheduled(spec, w, ids, [0, 1, 0, 1], [None, None, None, 1])
+    for cuts in (None, [13, 1, 1, 15], [2] * 15):
+        assert plain.rel_err(step_whole(runner, cache, ids, cuts), want) <= 1e-5
+
+
+# --------------------------------------------------------- a toy mixer with state
+
+
+@dataclass(frozen=True)
+class DecaySpec:
+    """y_t = s_t,  s_t = decay * s_{t-1} + W x_t  per sequence."""
+
+    kind: ClassVar[str] = "toy_decay"
+    decay: float
+
+
+def define_toy_mixer():
+    from shrike_amd.parts import Mixer, ParamSpec, StateSpec, register_mixer
+
+    class DecayMixer(Mixer):
+        def params(self):
+            return [ParamSpec(f"{self.name}.in_proj.weight", (self.width, self.width))]
+
+        def cache_spec(self):
+            return StateSpec((self.width,), "float32")
+
+        def load(self, tensors, runtime):
+            self.w = tensors[f"{self.name}.in_proj.weight"].float()
+
+        def forward(self, ctx, x, cache):
+            u = x.float() @ self.w.t()
+            out = torch.empty_like(u)
+            slots = ctx.state_slots.tolist()
+            start = 0
+            for s, n in enumerate(ctx.q_lens):
+                state = cache.state[slots[s]]
+                for t in range(start, start + n):
+                    state = self.spec.decay * state + u[t]
+                    out[t] = state
+                cache.state[slots[s]] = state
+                start += n
+            return out.to(x.dtype)
+
+    register_mixer("toy_decay", DecayMixer)
+
+
+def test_toy_mixer_with_state_is_registered_built_and_stepped():
+    from shrike_amd.engine.runner import StepEntry
+    from shrike_amd.parts import StateSpec
+
+    define_toy_mixer()
+    base = small_spec()
+    toy_block = replace(base.blocks[1], mixer=DecaySpec(decay=0.8), mixer_name="decay")
+    spec = replace(base, blocks=(base.blocks[0], toy_block))
+    w = cpu_weights(spec, seed=5)
+    assert "model.layers.1.decay.in_proj.weight" in w and "model.layers.1.self_attn.q_proj.weight" not in w
+    runner, model, cache = make_runner(spec, w)
+    assert model.cache_specs()[1] == StateSpec((48,), "float32")
+    assert len(cache.state_groups) == 1 and cache.state_groups[0].tensor.shape == (1, 8, 48)
+    assert cache.enable_prefix_caching is False
+
+    def want_for(ids):
+        cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
+        wd = {k: v.double() for k, v in w.items()}
+        n = len(ids)
+        cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+        x = plain.decoder_layer(cfg, wd, 0, wd["model.embed_tokens.weight"][torch.tensor(ids)], cos, sin)
+        p = "model.layers.1"
+        u = plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5) @ wd[f"{p}.decay.in_proj.weight"].t()
+        state, ys = torch.zeros(48, dtype=torch.float64), []
+        for t in range(n):
+            state = 0.8 * state + u[t]
+            ys.append(state)
+        x = x + torch.stack(ys)
+        h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
+        x = x + plain.swiglu(h, wd[f"{p}.mlp.gate_proj.weight"], wd[f"{p}.mlp.up_proj.weight"], wd[f"{p}.mlp.down_proj.weight"])
+        return plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+    g = torch.Generator().manual_seed(3)
+    a = torch.randint(0, 97, (19,), generator=g).tolist()
+    b = torch.randint(0, 97, (11,), generator=g).tolist()
+    assert plain.rel_err(step_whole(runner, cache, a), want_for(a)) <= 1e-5
+    assert plain.rel_err(step_whole(runner, cache, a, [4, 1, 1, 13]), want_for(a)) <= 1e-5
+    # two requests side by side, each with its own state slot; the slot of a
+    # finished request is handed out again and starts from zero
+    sa, sb = cache.new_sequence(), cache.new_sequence()
+    cache.append(sa, 0, 19)
+    cache.append(sb, 0, 11)
+    first = runner.step([StepEntry(sa, a[:7], 0, [6]), StepEntry(sb, b[:1], 0, [0])]).cpu().clone()
+    second = runner.step([StepEntry(sb, b[1:], 1, [9]), StepEntry(sa, a[7:], 7, [11])]).cpu().clone()
+    wa, wb = want_for(a), want_for(b)
+    got = torch.stack([first[0], first[1], second[0], second[1]]).double()
+    want = torch.stack([wa[6], wb[0], wb[10], wa[18]])
+    assert plain.rel_err(got, want) <= 1e-5
+    cache.free(sa)
+    cache.free(sb)
+    assert plain.rel_err(step_whole(runner, cache, b), wb) <= 1e-5

@@ -68,16 +68,16 @@ SEEDS = {"A": 11, "B": 23, "C": 37}
 PAGE_SIZES = {"A": 4, "B": 8, "C": 16}
 
 
-def make_model_dir(name: str, root=None, dtype: str = "float32") -> Path:
+def make_model_dir(name: str, root=None, dtype: str = "float32", mode: str = "reference") -> Path:
     """Writes the tiny model `name` with seeded random weights into a fresh
     temporary folder (or `root`/name) and returns the folder."""
     from shrike_amd.weights import write_model_folder
 
     if root is None:
         root = tempfile.mkdtemp(prefix="shrike_tiny_")
-    path = Path(root) / f"tiny_{name}_{dtype}"
+    path = Path(root) / f"tiny_{name}_{dtype}_{mode}"
     if not (path / "model.safetensors").is_file():
-        write_model_folder(dict(CONFIGS[name]), path, seed=SEEDS[name], dtype=dtype)
+        write_model_folder(dict(CONFIGS[name]), path, seed=SEEDS[name], dtype=dtype, mode=mode)
     return path
 
 
