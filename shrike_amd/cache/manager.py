@@ -3,9 +3,11 @@ one pool per group of layers with the same need, and slots for per-request
 state of fixed size.
 
 Layers whose mixers ask for the same PagedKVSpec form a group; a group has its
-own pool of pages, its own device tensor
-``[layers, 2, pages, kv_heads, page_size, head_dim]`` and, per request, its own
-block table.  A group with a window gives pages back as soon as no later query
+own pool of pages, its own device tensors (keys
+``[layers, pages, kv_heads, page_size, head_dim]``; values transposed,
+``[layers, pages, kv_heads, head_dim, page_size]``, so that the keys of a page
+are contiguous for every element) and, per request, its own block table.  A
+group with a window gives pages back as soon as no later query
 can reach them (table entry -1); all pages come back when the request ends.
 Layers whose mixers ask for a StateSpec form state groups: a tensor
 ``[layers, slots, *shape]`` indexed by the request's state slot.  Every request
@@ -52,7 +54,8 @@ class PageGroup:
         self.spec = spec
         self.layers: list[int] = []  # schedule positions that own a cache of this group
         self.pool = PagePool(num_pages)
-        self.tensor = None
+        self.k_tensor = None
+        self.v_tensor = None
 
 
 class StateGroup:
@@ -121,8 +124,12 @@ class CacheManager:
 
         for g in self.groups:
             s = g.spec
-            g.tensor = torch.zeros(
-                len(g.layers), 2, self.num_pages, s.num_kv_heads, self.page_size, s.head_dim,
+            g.k_tensor = torch.zeros(
+                len(g.layers), self.num_pages, s.num_kv_heads, self.page_size, s.head_dim,
+                dtype=dtype, device=device,
+            )
+            g.v_tensor = torch.zeros(
+                len(g.layers), self.num_pages, s.num_kv_heads, s.head_dim, self.page_size,
                 dtype=dtype, device=device,
             )
         for g in self.state_groups:
@@ -137,10 +144,10 @@ class CacheManager:
         family, gi, li = self._where[position]
         if family == "pages":
             g = self.groups[gi]
-            t = g.tensor
             return LayerCache(
                 group=gi, owned=not reader, page_size=self.page_size,
-                k_pool=None if t is None else t[li, 0], v_pool=None if t is None else t[li, 1],
+                k_pool=None if g.k_tensor is None else g.k_tensor[li],
+                v_pool=None if g.v_tensor is None else g.v_tensor[li],
                 window=g.spec.window,
             )
         g = self.state_groups[gi]

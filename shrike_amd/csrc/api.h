@@ -38,13 +38,24 @@ int shk_silu_mul(const void* gu, void* out, int dtype, int n, int inter, void* s
 int shk_gemm(const void* a, const void* w, const float* bias, void* out, int n, int m, int k,
              int lda, int ldo, int in_dtype, int out_dtype, int accumulate, void* stream);
 
+// wt = the tiled layout of the row-major bfloat16 matrix w[m, k] (see
+// gemm_bf16.hip): ceil(m/16) * ceil(k/32) tiles of 1 KiB.
+int shk_retile_weight(const void* w, int m, int k, void* wt, void* stream);
+
+// out[n, m] (+)= a[n, k] @ w^T + bias with w given in the tiled layout; a is
+// bfloat16 row-major with row stride lda; out is bfloat16 or float32.
+int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const float* bias, void* out, int n,
+                               int m, int k, int lda, int ldo, int out_dtype, int accumulate,
+                               void* stream);
+
 // Position encoding and cache write for the n tokens of a step.  qkv is
 // [n, (heads + 2*kv_heads) * head_dim]: queries, keys, values.  Queries and
 // keys are rotated by position (pairs (i, i + rot_dim/2), angle position *
 // inv_freq[i]); queries are rewritten in place; keys and values go to their
 // page slots: page = tables[token_seq[t] * table_stride + position / page_size].
-// Pools are [num_pages, kv_heads, page_size, head_dim].  rot_dim 0 rotates
-// nothing; write_kv 0 leaves the pools alone.
+// The key pool is [num_pages, kv_heads, page_size, head_dim]; the value pool is
+// stored transposed, [num_pages, kv_heads, head_dim, page_size].  rot_dim 0
+// rotates nothing; write_kv 0 leaves the pools alone.
 int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int head_dim,
                       int rot_dim, const float* inv_freq, const int32_t* positions,
                       const int32_t* token_seq, const int32_t* tables, int table_stride,
@@ -60,6 +71,30 @@ int shk_attention(const void* q, int q_stride, void* out, int dtype, int n, int 
                   const int32_t* tables, int table_stride, int num_seqs, const void* k_pool,
                   const void* v_pool, int page_size, int num_pages, int window, float scale,
                   void* stream);
+
+// 1 if the MFMA attention kernels take these shapes (head_dim a multiple of 32
+// up to 256, page_size a multiple of 16, at most 16 query heads per key/value
+// head, q rows 16-byte aligned); otherwise shk_attention serves them.
+int shk_attention_supports_mfma(int heads, int kv_heads, int head_dim, int page_size, int q_stride);
+
+// bfloat16 decode attention: sequence s has one query token, row s of q, at
+// positions[s].  Its keys are split over nsplit wavefronts per key/value head;
+// `partial` is float32 scratch of num_seqs * heads * nsplit * (head_dim + 2).
+int shk_attention_decode_bf16(const void* q, int q_stride, void* out, int num_seqs, int heads,
+                              int kv_heads, int head_dim, const int32_t* positions,
+                              const int32_t* tables, int table_stride, const void* k_pool,
+                              const void* v_pool, int page_size, int window, float scale,
+                              float* partial, int nsplit, void* stream);
+
+// bfloat16 attention for prompt portions, in tiles of 16 queries: tile i covers
+// queries tile_q0[i] .. +16 of sequence tile_seq[i]'s portion.  cu_q[s] is the
+// first token row of sequence s in q/out, ctx_lens[s] its length after the step.
+int shk_attention_prefill_bf16(const void* q, int q_stride, void* out, int num_tiles, int heads,
+                               int kv_heads, int head_dim, const int32_t* cu_q,
+                               const int32_t* ctx_lens, const int32_t* tile_seq,
+                               const int32_t* tile_q0, const int32_t* tables, int table_stride,
+                               const void* k_pool, const void* v_pool, int page_size, int window,
+                               float scale, void* stream);
 
 // out[r] = lowest index of the largest value of logits[r, :vocab].
 int shk_argmax(const float* logits, int32_t* out, int rows, int vocab, int ld, void* stream);

@@ -26,7 +26,7 @@ __global__ void __launch_bounds__(kAttnThreads)
                              int page_size, int num_pages, int window, float scale) {
   __shared__ float qs[kMaxHeadDim];
   __shared__ float probs[kAttnThreads];
-  __shared__ int32_t rows[kAttnThreads];  // cache row of each key of the tile, -1 if masked
+  __shared__ int32_t rows[kAttnThreads];  // key-cache row of each key of the tile, -1 if masked
   __shared__ float scratch[16];
   __shared__ float partial[kAttnThreads];
 
@@ -73,7 +73,11 @@ __global__ void __launch_bounds__(kAttnThreads)
       const int count = (pos - j0 + 1 < kAttnThreads) ? pos - j0 + 1 : kAttnThreads;
       for (int jj = g; jj < count; jj += groups) {
         const int32_t r = rows[jj];
-        if (r >= 0) a = fmaf(probs[jj], to_float(v_pool[static_cast<size_t>(r) * head_dim + d]), a);
+        if (r < 0) continue;
+        // values are stored [page][kv head][head_dim][page_size]
+        const size_t v_at =
+            (static_cast<size_t>(r / page_size) * head_dim + d) * page_size + r % page_size;
+        a = fmaf(probs[jj], to_float(v_pool[v_at]), a);
       }
       acc = acc * alpha + a;
     }

@@ -1,0 +1,421 @@
+// bfloat16 attention over the paged cache on the MFMA units (gfx950).
+//
+// One wavefront owns a tile of 16 "rows" that share a key/value head of one
+// sequence: for a prompt portion the rows are 16 consecutive queries of one
+// query head; for a decoded token they are the query heads of one group
+// (padded to 16).  The wavefront walks its key range in chunks of 32 keys:
+//
+//   S = Q K^T      two 16x16 tiles, v_mfma_f32_16x16x32_bf16 over head_dim;
+//                  K rows are read straight from the page ([slot][head_dim])
+//   softmax        running maximum and sum per row in float32, exp in float32
+//   O += P V       P goes through LDS into operand layout; V is stored
+//                  transposed in the cache ([head_dim][slot]), so 8 keys of one
+//                  element are one 16-byte load
+//
+// Decode splits a sequence's keys over several wavefronts; each writes an
+// unnormalised partial (O, max, sum) and attention_merge_kernel combines them
+// in a fixed order.  Head sizes: multiples of 32 up to 256; page sizes:
+// multiples of 16; up to 16 query heads per key/value head.  Other shapes are
+// served by the general kernel.
+#include "api.h"
+#include "common.h"
+
+namespace shk {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+union AFrag {
+  uint4 u;
+  bf16x8 v;
+  uint16_t h[8];
+};
+
+constexpr int kPStride = 40;  // bf16 elements per row of the P tile in LDS (32 + padding)
+
+struct TileArgs {
+  const int32_t* table;  // block table of the sequence
+  const bf16* k_pool;    // [pages][kv_heads][page_size][D]
+  const bf16* v_pool;    // [pages][kv_heads][D][page_size]
+  int page_size;
+  int kv_heads;
+  int kvh;
+  float scale;
+};
+
+// Walks keys [key_begin, key_end) (key_begin a multiple of 32) for 16 rows.
+// qf: the rows' queries as A operands.  row_pos / row_lo: for this lane's four
+// accumulator rows (4*(lane/16) + r), the last and first key each may read.
+// pos_max / lo_min: the same bounds over all 16 rows.
+template <int D>
+__device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf)[D / 32],
+                                            const int (&row_pos)[4], const int (&row_lo)[4],
+                                            int pos_max, int lo_min, int key_begin, int key_end,
+                                            f32x4 (&o)[D / 16], float (&m)[4], float (&l)[4],
+                                            uint16_t* p_lds) {
+  const int lane = threadIdx.x % kWave;
+  const int j = lane % 16, kg = lane / 16;
+  const int ps = ta.page_size;
+  const size_t head_elems = static_cast<size_t>(ps) * D;  // one kv head of one page
+
+  for (int kb = key_begin; kb < key_end; kb += 32) {
+    // ---- S = Q K^T for two tiles of 16 keys
+    f32x4 s[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int key0 = kb + tt * 16;
+      if (key0 > pos_max || key0 + 15 < lo_min) continue;  // no row reads this tile
+      const int page = ta.table[key0 / ps];
+      const bf16* krow = ta.k_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
+                         static_cast<size_t>(key0 % ps + j) * D + kg * 8;
+      AFrag kf[D / 32];
+#pragma unroll
+      for (int ds = 0; ds < D / 32; ++ds) kf[ds].u = *reinterpret_cast<const uint4*>(krow + ds * 32);
+#pragma unroll
+      for (int ds = 0; ds < D / 32; ++ds)
+        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ds].v, kf[ds].v, s[tt], 0, 0, 0);
+    }
+
+    // ---- mask, running maximum and sum (lane holds key kb + tt*16 + j for rows 4*kg + r)
+    float p[2][4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float sc[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        const int key = kb + tt * 16 + j;
+        const bool keep = key <= row_pos[r] && key >= row_lo[r];
+        sc[tt] = keep ? s[tt][r] * ta.scale : -INFINITY;
+      }
+      float mx = fmaxf(sc[0], sc[1]);
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+      const float m_new = fmaxf(m[r], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __expf(m[r] - m_safe);
+      p[0][r] = __expf(sc[0] - m_safe);
+      p[1][r] = __expf(sc[1] - m_safe);
+      float sum = p[0][r] + p[1][r];
+#pragma unroll
+      for (int off = 1; off < 16; off <<= 1) sum += __shfl_xor(sum, off, kWave);
+      l[r] = l[r] * alpha + sum;
+      m[r] = m_new;
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db) o[db][r] *= alpha;
+    }
+
+    // ---- P through LDS into A-operand layout: rows 16, keys 32
+    __syncthreads();  // the previous chunk's reads are done (one wavefront per workgroup)
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        p_lds[(kg * 4 + r) * kPStride + tt * 16 + j] = bf16_bits(p[tt][r]);
+    __syncthreads();
+    AFrag pf;
+    pf.u = *reinterpret_cast<const uint4*>(p_lds + j * kPStride + kg * 8);
+
+    // ---- O += P V: this lane supplies keys kb + 8*kg .. +8 of element db*16 + j
+    const int g0 = kb + kg * 8;
+    const bool live = g0 <= pos_max && g0 + 7 >= lo_min;
+    const bf16* vcol = nullptr;
+    if (live) {
+      const int page = ta.table[g0 / ps];
+      vcol = ta.v_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
+             static_cast<size_t>(j) * ps + g0 % ps;
+    }
+    // keys outside [lo_min, pos_max] carry weight 0 but may hold anything: zero them
+    uint4 keep_bits = make_uint4(~0u, ~0u, ~0u, ~0u);
+    if (live && (g0 < lo_min || g0 + 7 > pos_max)) {
+      uint32_t w[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const bool a = g0 + 2 * e >= lo_min && g0 + 2 * e <= pos_max;
+        const bool b = g0 + 2 * e + 1 >= lo_min && g0 + 2 * e + 1 <= pos_max;
+        w[e] = (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
+      }
+      keep_bits = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      AFrag vf;
+      vf.u = make_uint4(0, 0, 0, 0);
+      if (live) {
+        vf.u = *reinterpret_cast<const uint4*>(vcol + static_cast<size_t>(db) * 16 * ps);
+        vf.u.x &= keep_bits.x;
+        vf.u.y &= keep_bits.y;
+        vf.u.z &= keep_bits.z;
+        vf.u.w &= keep_bits.w;
+      }
+      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, o[db], 0, 0, 0);
+    }
+  }
+}
+
+// ------------------------------------------------------------------- decode
+// grid (kv_heads, sequences, splits), one wavefront per workgroup.
+
+template <int D>
+__global__ void __launch_bounds__(kWave)
+    attention_decode_kernel(const bf16* __restrict__ q, int q_stride, int heads, int kv_heads,
+                            const int32_t* __restrict__ positions,
+                            const int32_t* __restrict__ tables, int table_stride,
+                            const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+                            int page_size, int window, float scale, float* __restrict__ partial,
+                            int nsplit) {
+  __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * kPStride];
+  const int kvh = blockIdx.x, seq = blockIdx.y, z = blockIdx.z;
+  const int lane = threadIdx.x, j = lane % 16, kg = lane / 16;
+  const int group = heads / kv_heads;
+  // decode sequences come first in the step: token index == sequence index
+  const int pos = positions[seq];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+
+  // this split's keys: chunks of 32 from the chunk that holds `lo`
+  const int first = lo & ~31;
+  const int chunks = (pos - first) / 32 + 1;
+  const int per = (chunks + nsplit - 1) / nsplit;
+  const int key_begin = first + z * per * 32;
+  int key_end = key_begin + per * 32;
+  if (key_end > pos + 1) key_end = pos + 1;
+
+  float m[4], l[4];
+  f32x4 o[D / 16];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) m[r] = -INFINITY, l[r] = 0.f;
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  if (key_begin <= pos) {
+    AFrag qf[D / 32];
+    const bf16* qrow = q + static_cast<size_t>(seq) * q_stride +
+                       static_cast<size_t>(kvh * group + j) * D + kg * 8;
+#pragma unroll
+    for (int ds = 0; ds < D / 32; ++ds) {
+      qf[ds].u = make_uint4(0, 0, 0, 0);
+      if (j < group) qf[ds].u = *reinterpret_cast<const uint4*>(qrow + ds * 32);
+    }
+    const int row_pos[4] = {pos, pos, pos, pos};
+    const int row_lo[4] = {lo, lo, lo, lo};
+    TileArgs ta{tables + static_cast<size_t>(seq) * table_stride, k_pool, v_pool, page_size,
+                kv_heads, kvh, scale};
+    attend_tile<D>(ta, qf, row_pos, row_lo, pos, lo, key_begin, key_end, o, m, l, p_lds);
+  }
+
+  // partial[seq][head][split] = {O[D], max, sum}; lane holds element db*16 + j of rows 4*kg + r
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int hrow = kg * 4 + r;
+    if (hrow >= group) continue;
+    float* dst = partial + ((static_cast<size_t>(seq) * heads + kvh * group + hrow) * nsplit + z) *
+                               (D + 2);
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) dst[db * 16 + j] = o[db][r];
+    if (j == 0) {
+      dst[D] = m[r];
+      dst[D + 1] = l[r];
+    }
+  }
+}
+
+// out[seq][head][:] = sum_z exp(m_z - M) O_z / sum_z exp(m_z - M) l_z, splits in order.
+__global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
+                                       int head_dim, int nsplit) {
+  const size_t row = blockIdx.x;  // seq * heads + head
+  const float* src = partial + row * nsplit * (head_dim + 2);
+  float mx = -INFINITY;
+  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, src[z * (head_dim + 2) + head_dim]);
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float num = 0.f, den = 0.f;
+    for (int z = 0; z < nsplit; ++z) {
+      const float* pz = src + z * (head_dim + 2);
+      const float mz = pz[head_dim];
+      if (mz == -INFINITY) continue;
+      const float f = __expf(mz - mx);
+      num += f * pz[d];
+      den += f * pz[head_dim + 1];
+    }
+    out[row * head_dim + d] = from_float<bf16>(num / den);
+  }
+}
+
+// ------------------------------------------------------------------ prefill
+// grid (query tiles of 16 over all portions, heads), one wavefront per
+// workgroup.  tile_seq / tile_q0: for each tile its sequence and the offset of
+// its first query inside the sequence's portion.
+
+template <int D>
+__global__ void __launch_bounds__(kWave)
+    attention_prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+                             int heads, int kv_heads, const int32_t* __restrict__ cu_q,
+                             const int32_t* __restrict__ ctx_lens,
+                             const int32_t* __restrict__ tile_seq,
+                             const int32_t* __restrict__ tile_q0,
+                             const int32_t* __restrict__ tables, int table_stride,
+                             const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+                             int page_size, int window, float scale) {
+  __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * kPStride];
+  const int tile = blockIdx.x, head = blockIdx.y;
+  const int lane = threadIdx.x, j = lane % 16, kg = lane / 16;
+  const int seq = tile_seq[tile], q0 = tile_q0[tile];
+  const int tok0 = cu_q[seq], q_len = cu_q[seq + 1] - tok0;
+  const int start = ctx_lens[seq] - q_len;  // position of the portion's first token
+  const int kvh = head / (heads / kv_heads);
+  const int rows = (q_len - q0 < 16) ? q_len - q0 : 16;
+
+  AFrag qf[D / 32];
+  const bf16* qrow = q + static_cast<size_t>(tok0 + q0 + j) * q_stride +
+                     static_cast<size_t>(head) * D + kg * 8;
+#pragma unroll
+  for (int ds = 0; ds < D / 32; ++ds) {
+    qf[ds].u = make_uint4(0, 0, 0, 0);
+    if (j < rows) qf[ds].u = *reinterpret_cast<const uint4*>(qrow + ds * 32);
+  }
+
+  int row_pos[4], row_lo[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int qi = kg * 4 + r;
+    row_pos[r] = (qi < rows) ? start + q0 + qi : -1;  // rows past the portion read nothing
+    row_lo[r] = (window > 0 && row_pos[r] - window + 1 > 0) ? row_pos[r] - window + 1 : 0;
+  }
+  const int pos_min = start + q0, pos_max = start + q0 + rows - 1;
+  const int lo_min = (window > 0 && pos_min - window + 1 > 0) ? pos_min - window + 1 : 0;
+
+  float m[4], l[4];
+  f32x4 o[D / 16];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) m[r] = -INFINITY, l[r] = 0.f;
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  TileArgs ta{tables + static_cast<size_t>(seq) * table_stride, k_pool, v_pool, page_size,
+              kv_heads, kvh, scale};
+  attend_tile<D>(ta, qf, row_pos, row_lo, pos_max, lo_min, lo_min & ~31, pos_max + 1, o, m, l,
+                 p_lds);
+
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int qi = kg * 4 + r;
+    if (qi >= rows) continue;
+    bf16* dst = out + static_cast<size_t>(tok0 + q0 + qi) * heads * D + static_cast<size_t>(head) * D;
+    const float inv = 1.f / l[r];
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) dst[db * 16 + j] = from_float<bf16>(o[db][r] * inv);
+  }
+}
+
+template <int D>
+static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, int heads,
+                          int kv_heads, const int32_t* positions, const int32_t* tables,
+                          int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
+                          int window, float scale, float* partial, int nsplit) {
+  attention_decode_kernel<D><<<grid, kWave, 0, s>>>(q, q_stride, heads, kv_heads, positions, tables,
+                                                    table_stride, k_pool, v_pool, page_size,
+                                                    window, scale, partial, nsplit);
+}
+
+template <int D>
+static void launch_prefill(dim3 grid, hipStream_t s, const bf16* q, int q_stride, bf16* out,
+                           int heads, int kv_heads, const int32_t* cu_q, const int32_t* ctx_lens,
+                           const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tables,
+                           int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
+                           int window, float scale) {
+  attention_prefill_kernel<D><<<grid, kWave, 0, s>>>(q, q_stride, out, heads, kv_heads, cu_q,
+                                                     ctx_lens, tile_seq, tile_q0, tables,
+                                                     table_stride, k_pool, v_pool, page_size,
+                                                     window, scale);
+}
+
+}  // namespace shk
+
+using namespace shk;
+
+#define SHK_DISPATCH_D(D, CALL)                                                         \
+  switch (D) {                                                                          \
+    case 32: CALL(32); break;                                                           \
+    case 64: CALL(64); break;                                                           \
+    case 96: CALL(96); break;                                                           \
+    case 128: CALL(128); break;                                                         \
+    case 160: CALL(160); break;                                                         \
+    case 192: CALL(192); break;                                                         \
+    case 224: CALL(224); break;                                                         \
+    case 256: CALL(256); break;                                                         \
+    default: break;                                                                     \
+  }
+
+static int check_mfma_shapes(const char* who, int heads, int kv_heads, int head_dim, int page_size,
+                             int q_stride) {
+  SHK_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0,
+              "%s: heads=%d must be a positive multiple of kv_heads=%d", who, heads, kv_heads);
+  SHK_REQUIRE(head_dim % 32 == 0 && head_dim >= 32 && head_dim <= 256,
+              "%s: head_dim %d is not a multiple of 32 in 32..256", who, head_dim);
+  SHK_REQUIRE(page_size > 0 && page_size % 16 == 0, "%s: page_size %d is not a multiple of 16", who,
+              page_size);
+  SHK_REQUIRE(q_stride % 8 == 0, "%s: q_stride %d is not a multiple of 8", who, q_stride);
+  return 0;
+}
+
+extern "C" int shk_attention_supports_mfma(int heads, int kv_heads, int head_dim, int page_size,
+                                           int q_stride) {
+  return heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && heads / kv_heads <= 16 &&
+         head_dim % 32 == 0 && head_dim >= 32 && head_dim <= 256 && page_size > 0 &&
+         page_size % 16 == 0 && q_stride % 8 == 0;
+}
+
+extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out, int num_seqs,
+                                         int heads, int kv_heads, int head_dim,
+                                         const int32_t* positions, const int32_t* tables,
+                                         int table_stride, const void* k_pool, const void* v_pool,
+                                         int page_size, int window, float scale, float* partial,
+                                         int nsplit, void* stream) {
+  if (check_mfma_shapes("attention_decode", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
+  SHK_REQUIRE(heads / kv_heads <= 16, "attention_decode: at most 16 query heads per key/value head");
+  SHK_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && nsplit >= 1 && nsplit <= 65535,
+              "attention_decode: bad sizes num_seqs=%d nsplit=%d", num_seqs, nsplit);
+  if (num_seqs == 0) return 0;
+  SHK_REQUIRE(q && out && positions && tables && k_pool && v_pool && partial && table_stride > 0,
+              "attention_decode: null pointer");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q is not 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(kv_heads, num_seqs, nsplit);
+#define CALL(D)                                                                              \
+  launch_decode<D>(grid, s, static_cast<const bf16*>(q), q_stride, heads, kv_heads, positions, \
+                   tables, table_stride, static_cast<const bf16*>(k_pool),                   \
+                   static_cast<const bf16*>(v_pool), page_size, window, scale, partial, nsplit)
+  SHK_DISPATCH_D(head_dim, CALL)
+#undef CALL
+  SHK_LAUNCH_CHECK("attention_decode");
+  attention_merge_kernel<<<num_seqs * heads, head_dim <= 64 ? 64 : 128, 0, s>>>(
+      partial, static_cast<bf16*>(out), head_dim, nsplit);
+  SHK_LAUNCH_CHECK("attention_merge");
+  return 0;
+}
+
+extern "C" int shk_attention_prefill_bf16(const void* q, int q_stride, void* out, int num_tiles,
+                                          int heads, int kv_heads, int head_dim,
+                                          const int32_t* cu_q, const int32_t* ctx_lens,
+                                          const int32_t* tile_seq, const int32_t* tile_q0,
+                                          const int32_t* tables, int table_stride,
+                                          const void* k_pool, const void* v_pool, int page_size,
+                                          int window, float scale, void* stream) {
+  if (check_mfma_shapes("attention_prefill", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
+  SHK_REQUIRE(num_tiles >= 0 && heads <= 65535, "attention_prefill: bad sizes");
+  if (num_tiles == 0) return 0;
+  SHK_REQUIRE(q && out && cu_q && ctx_lens && tile_seq && tile_q0 && tables && k_pool && v_pool &&
+                  table_stride > 0,
+              "attention_prefill: null pointer");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_prefill: q is not 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(num_tiles, heads);
+#define CALL(D)                                                                              \
+  launch_prefill<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
+                    heads, kv_heads, cu_q, ctx_lens, tile_seq, tile_q0, tables, table_stride, \
+                    static_cast<const bf16*>(k_pool), static_cast<const bf16*>(v_pool),      \
+                    page_size, window, scale)
+  SHK_DISPATCH_D(head_dim, CALL)
+#undef CALL
+  SHK_LAUNCH_CHECK("attention_prefill");
+  return 0;
+}

@@ -32,8 +32,9 @@ __global__ void __launch_bounds__(256)
 
   T* row = qkv + static_cast<size_t>(t) * (heads + 2 * kv_heads) * head_dim;
   size_t slot_row = 0;  // index of this token's [head_dim] row for kv head 0
+  int page = 0;
   if (write_kv) {
-    const int page = tables[static_cast<size_t>(token_seq[t]) * table_stride + pos / page_size];
+    page = tables[static_cast<size_t>(token_seq[t]) * table_stride + pos / page_size];
     // The host builds tables that cover every position of the step; a page id
     // outside the pool would be a host bug, and is never dereferenced.
     if (page < 0 || page >= num_pages) write_kv = 0;
@@ -66,12 +67,12 @@ __global__ void __launch_bounds__(256)
     const int h = idx / tail, i = rot_dim + idx % tail;
     k_pool[(slot_row + h * head_rows) * head_dim + i] = krow[h * head_dim + i];
   }
-  // values: copy
+  // values: stored transposed, [page][kv head][head_dim][page_size], so that the
+  // keys of a page are contiguous for every element (the operand layout of P.V)
   const T* vrow = krow + kv_heads * head_dim;
-  for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x) {
-    const int h = idx / head_dim, i = idx % head_dim;
-    v_pool[(slot_row + h * head_rows) * head_dim + i] = vrow[h * head_dim + i];
-  }
+  const size_t vbase = static_cast<size_t>(page) * kv_heads * head_dim * page_size + pos % page_size;
+  for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x)
+    v_pool[vbase + static_cast<size_t>(idx) * page_size] = vrow[idx];
 }
 
 }  // namespace shk

@@ -12,6 +12,8 @@ first, then prompt portions, each sequence's tokens contiguous):
                                                sequence's first portion
   block_tables[g][S, blocks_g]                 page ids per page group
   out_rows[R]                                  rows whose logits are wanted
+  tile_seq[T]  tile_q0[T]                      prompt portions cut into tiles of 16
+                                               queries: sequence and first query
 
 The reference builds the same information per step as Python lists and one
 tensor per sequence (shrike/engine/model_runner.py:205-248).
@@ -65,6 +67,10 @@ class StepContext:
     ctx_lens_host: list[int] = field(default_factory=list)
     max_q_len: int = 0
     max_ctx_len: int = 0
+    max_decode_ctx: int = 0  # longest context among the single-token sequences
+    tile_seq: torch.Tensor | None = None
+    tile_q0: torch.Tensor | None = None
+    num_prefill_tiles: int = 0
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)

@@ -107,8 +107,16 @@ class ModelRunner:
                 t[k, : len(row)] = row
             tables.append(t)
 
+        # prompt portions in tiles of 16 queries for the MFMA attention kernel
+        tile_counts = -(-q_lens[num_decode:] // 16)
+        tile_seq = np.repeat(np.arange(num_decode, num_seqs), tile_counts)
+        tile_first = np.zeros(num_seqs - num_decode + 1, dtype=np.int64)
+        np.cumsum(tile_counts, out=tile_first[1:])
+        tile_q0 = (np.arange(int(tile_counts.sum())) - tile_first[tile_seq - num_decode]) * 16
+
         parts = [token_ids, positions, token_seq, cu_q, ctx_lens, state_slots, fresh,
-                 np.asarray(out_rows, dtype=np.int64)] + [t.reshape(-1) for t in tables]
+                 np.asarray(out_rows, dtype=np.int64), tile_seq, tile_q0]
+        parts += [t.reshape(-1) for t in tables]
         sizes = [p.size for p in parts]
         total = int(sum(sizes))
         if self._pinned_free is not None:
@@ -130,9 +138,11 @@ class ModelRunner:
             num_tokens=num_tokens, num_seqs=num_seqs, num_decode=num_decode,
             token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
             ctx_lens=views[4], state_slots=views[5], fresh=views[6], out_rows=views[7],
-            block_tables=[v.view(num_seqs, t.shape[1]) for v, t in zip(views[8:], tables)],
+            tile_seq=views[8], tile_q0=views[9], num_prefill_tiles=int(tile_seq.size),
+            block_tables=[v.view(num_seqs, t.shape[1]) for v, t in zip(views[10:], tables)],
             q_lens=q_lens.tolist(), ctx_lens_host=ctx_lens.tolist(),
             max_q_len=int(q_lens.max()), max_ctx_len=int(ctx_lens.max()),
+            max_decode_ctx=int(ctx_lens[:num_decode].max()) if num_decode else 0,
         )
 
     # -------------------------------------------------------------------- step

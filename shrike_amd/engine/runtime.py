@@ -1,9 +1,11 @@
-"""The runtime a model is loaded into: device, compute dtype, and the choice
-of kernel for each matrix product and attention call.
+"""The runtime a model is loaded into: device, compute dtype, how matrices are
+held, and the choice of kernel for each matrix product and attention call.
 
 float32: every product runs in the general float32 kernel (fused multiply-add,
 no matrix mode of reduced precision) and attention in the general kernel.
-bfloat16: the serving kernels.
+bfloat16: weights are also held in the MFMA operand layout; products with at
+most 64 rows stream them once through the skinny MFMA kernel; attention runs
+on the MFMA kernels where the shapes allow, else in the general kernel.
 """
 
 from __future__ import annotations
@@ -11,6 +13,19 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
+
+SKINNY_ROWS = 64  # most rows of a step that the weight-streaming kernel takes
+
+
+class LinearWeight:
+    """A weight matrix [rows, cols] as the kernels want it."""
+
+    __slots__ = ("rows", "cols", "dense", "tiled")
+
+    def __init__(self, dense: torch.Tensor, tiled: torch.Tensor | None):
+        self.rows, self.cols = dense.shape
+        self.dense = dense
+        self.tiled = tiled
 
 
 class Runtime:
@@ -20,15 +35,45 @@ class Runtime:
             raise ValueError(f"compute dtype must be bfloat16 or float32, got {dtype}")
         self.dtype = dtype
 
-    def linear(self, x, w, out, bias=None, accumulate=False) -> None:
+    def weight(self, w: torch.Tensor) -> LinearWeight:
+        """Takes a row-major [out, in] matrix in the compute dtype."""
+        w = w.contiguous()
+        tiled = ops.retile_weight(w) if self.dtype == torch.bfloat16 else None
+        return LinearWeight(w, tiled)
+
+    def linear(self, x, w: LinearWeight, out, bias=None, accumulate=False) -> None:
         """out (+)= x @ w.T + bias."""
-        ops.gemm(x, w, out, bias=bias, accumulate=accumulate)
+        if w.tiled is not None and x.shape[0] <= SKINNY_ROWS:
+            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, bias=bias, accumulate=accumulate)
+        else:
+            ops.gemm(x, w.dense, out, bias=bias, accumulate=accumulate)
 
     def attend(self, ctx, qkv, out, spec, tables, cache) -> None:
         """Attention of every token of the step over its sequence's cache."""
-        q = qkv[:, : spec.num_heads * spec.head_dim]
-        ops.attention(
-            q, out, spec.num_heads, spec.num_kv_heads, spec.head_dim, ctx.positions,
-            ctx.token_seq, tables, cache.k_pool, cache.v_pool, cache.page_size,
-            spec.window, spec.scale,
-        )
+        h, hkv, d = spec.num_heads, spec.num_kv_heads, spec.head_dim
+        q = qkv[:, : h * d]
+        if self.dtype == torch.bfloat16 and ops.attention_supports_mfma(
+            h, hkv, d, cache.page_size, qkv.stride(0)
+        ):
+            if ctx.num_decode:
+                nsplit = decode_splits(ctx.num_decode, hkv, ctx.max_decode_ctx)
+                partial = ctx.buffer("attn_partial", (ctx.num_decode * h * nsplit * (d + 2),),
+                                     torch.float32)
+                ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
+                                     cache.k_pool, cache.v_pool, cache.page_size, spec.window,
+                                     spec.scale, partial, nsplit)
+            if ctx.num_prefill_tiles:
+                ops.attention_prefill(q, out, ctx.num_prefill_tiles, h, hkv, d, ctx.cu_q,
+                                      ctx.ctx_lens, ctx.tile_seq, ctx.tile_q0, tables, cache.k_pool,
+                                      cache.v_pool, cache.page_size, spec.window, spec.scale)
+            return
+        ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.k_pool,
+                      cache.v_pool, cache.page_size, spec.window, spec.scale)
+
+
+def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
+    """Wavefronts per (sequence, key/value head): enough to fill the chip
+    (about 2048 in all), each with at least 128 keys."""
+    want = -(-2048 // max(1, num_seqs * kv_heads))
+    most = max(1, max_ctx // 128)
+    return max(1, min(want, most, 64))

@@ -109,22 +109,73 @@ def gemm(a, w, out, bias=None, accumulate=False) -> None:
     )
 
 
+def tiled_numel(m: int, k: int) -> int:
+    """bfloat16 elements of the tiled layout of an [m, k] matrix."""
+    return -(-m // 16) * -(-k // 32) * 512
+
+
+def retile_weight(w: torch.Tensor) -> torch.Tensor:
+    """The MFMA operand layout of a row-major bfloat16 [m, k] matrix (a flat tensor)."""
+    if w.dim() != 2 or not w.is_contiguous() or w.dtype != torch.bfloat16:
+        raise KernelError("retile_weight: expected a contiguous bfloat16 matrix")
+    m, k = w.shape
+    wt = torch.empty(tiled_numel(m, k), dtype=torch.bfloat16, device=w.device)
+    check(load().shk_retile_weight(_dev(w, "w"), m, k, _dev(wt, "wt"), _stream()))
+    return wt
+
+
+def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False) -> None:
+    """out (+)= a @ w.T + bias for at most 64 rows of a; wt = retile_weight(w)."""
+    _rows(a, "gemm a")
+    _rows(out, "gemm out")
+    n = a.shape[0]
+    if a.shape[1] != k or a.dtype != torch.bfloat16:
+        raise KernelError(f"gemm_tiled_weight: a must be bfloat16 [n, {k}], got {tuple(a.shape)}")
+    if out.shape != (n, m):
+        raise KernelError(f"gemm_tiled_weight: out must be [{n}, {m}], got {tuple(out.shape)}")
+    if wt.numel() != tiled_numel(m, k) or wt.dtype != torch.bfloat16:
+        raise KernelError("gemm_tiled_weight: wt is not the tiled layout of an [m, k] matrix")
+    if bias is not None and bias.numel() != m:
+        raise KernelError(f"gemm_tiled_weight: bias has {bias.numel()} elements, m is {m}")
+    check(
+        load().shk_gemm_bf16_tiled_weight(
+            _dev(a, "a"), _dev(wt, "wt"),
+            None if bias is None else _dev(bias, "bias", torch.float32),
+            _dev(out, "out"), n, m, k, a.stride(0), out.stride(0), dtype_code(out.dtype),
+            int(bool(accumulate)), _stream(),
+        )
+    )
+
+
+def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size) -> None:
+    """Keys [pages, kv_heads, page_size, head_dim]; values transposed
+    [pages, kv_heads, head_dim, page_size]."""
+    pages = k_pool.shape[0]
+    if tuple(k_pool.shape) != (pages, kv_heads, page_size, head_dim):
+        raise KernelError(f"{who}: key pool must be [pages, {kv_heads}, {page_size}, {head_dim}], "
+                          f"got {tuple(k_pool.shape)}")
+    if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_size):
+        raise KernelError(f"{who}: value pool must be [pages, {kv_heads}, {head_dim}, {page_size}], "
+                          f"got {tuple(v_pool.shape)}")
+    if k_pool.dtype != q.dtype or v_pool.dtype != q.dtype:
+        raise KernelError(f"{who}: pools and queries differ in dtype")
+    if not (k_pool.is_contiguous() and v_pool.is_contiguous() and tables.is_contiguous()):
+        raise KernelError(f"{who}: pools and tables must be contiguous")
+    if tables.dim() != 2:
+        raise KernelError(f"{who}: tables must be [sequences, blocks]")
+
+
 def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, token_seq,
                   tables, k_pool, v_pool, page_size, write_kv=True) -> None:
     """Rotate q and k of qkv [n, (heads + 2 kv_heads) head_dim] in float32 and put
-    k, v into their pages; pools are [pages, kv_heads, page_size, head_dim]."""
+    k, v into their pages (keys [pages, kv_heads, page_size, head_dim], values
+    transposed [pages, kv_heads, head_dim, page_size])."""
     n = qkv.shape[0]
     if not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
         raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim]")
     num_pages = 0
     if write_kv:
-        want = (k_pool.shape[0], kv_heads, page_size, head_dim)
-        if tuple(k_pool.shape) != want or tuple(v_pool.shape) != want:
-            raise KernelError(f"rope_kv_store: pools must be {want}, got {tuple(k_pool.shape)}")
-        if k_pool.dtype != qkv.dtype or v_pool.dtype != qkv.dtype:
-            raise KernelError("rope_kv_store: pools and qkv differ in dtype")
-        if not (k_pool.is_contiguous() and v_pool.is_contiguous() and tables.is_contiguous()):
-            raise KernelError("rope_kv_store: pools and tables must be contiguous")
+        _check_pools("rope_kv_store", qkv, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
         num_pages = k_pool.shape[0]
     check(
         load().shk_rope_kv_store(
@@ -148,13 +199,7 @@ def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k
     n = q.shape[0]
     if out.shape != (n, heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
         raise KernelError("attention: out must be contiguous [n, heads*head_dim] of q's dtype")
-    want = (k_pool.shape[0], kv_heads, page_size, head_dim)
-    if tuple(k_pool.shape) != want or tuple(v_pool.shape) != want:
-        raise KernelError(f"attention: pools must be {want}, got {tuple(k_pool.shape)}")
-    if k_pool.dtype != q.dtype or v_pool.dtype != q.dtype:
-        raise KernelError("attention: pools and q differ in dtype")
-    if not (k_pool.is_contiguous() and v_pool.is_contiguous() and tables.is_contiguous()):
-        raise KernelError("attention: pools and tables must be contiguous")
+    _check_pools("attention", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
     check(
         load().shk_attention(
             _dev(q, "q"), q.stride(0), _dev(out, "out"), dtype_code(q.dtype), n, heads, kv_heads,
@@ -162,6 +207,56 @@ def attention(q, out, heads, kv_heads, head_dim, positions, token_seq, tables, k
             _dev(token_seq, "token_seq", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], tables.shape[0], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"),
             page_size, k_pool.shape[0], int(window or 0), float(scale), _stream(),
+        )
+    )
+
+
+def attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride) -> bool:
+    return bool(load().shk_attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride))
+
+
+def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tables, k_pool, v_pool,
+                     page_size, window, scale, partial, nsplit) -> None:
+    """bfloat16 MFMA attention for the first num_seqs rows of q, one token per sequence."""
+    _rows(q, "attention_decode q")
+    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("attention_decode: bfloat16 only")
+    if q.shape[0] < num_seqs or tables.shape[0] < num_seqs or positions.shape[0] < num_seqs:
+        raise KernelError("attention_decode: fewer rows than sequences")
+    if out.shape[0] < num_seqs or out.shape[1] != heads * head_dim or not out.is_contiguous():
+        raise KernelError("attention_decode: out must be contiguous [>= num_seqs, heads*head_dim]")
+    _check_pools("attention_decode", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
+    if partial.numel() < num_seqs * heads * nsplit * (head_dim + 2):
+        raise KernelError("attention_decode: partial scratch is too small")
+    check(
+        load().shk_attention_decode_bf16(
+            _dev(q, "q"), q.stride(0), _dev(out, "out"), num_seqs, heads, kv_heads, head_dim,
+            _dev(positions, "positions", torch.int32), _dev(tables, "tables", torch.int32),
+            tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size,
+            int(window or 0), float(scale), _dev(partial, "partial", torch.float32), nsplit,
+            _stream(),
+        )
+    )
+
+
+def attention_prefill(q, out, num_tiles, heads, kv_heads, head_dim, cu_q, ctx_lens, tile_seq, tile_q0,
+                      tables, k_pool, v_pool, page_size, window, scale) -> None:
+    """bfloat16 MFMA attention for prompt portions, in tiles of 16 queries."""
+    _rows(q, "attention_prefill q")
+    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("attention_prefill: bfloat16 only")
+    if out.shape != (q.shape[0], heads * head_dim) or not out.is_contiguous():
+        raise KernelError("attention_prefill: out must be contiguous [n, heads*head_dim]")
+    if tile_seq.shape[0] < num_tiles or tile_q0.shape[0] < num_tiles:
+        raise KernelError("attention_prefill: tile arrays are shorter than num_tiles")
+    _check_pools("attention_prefill", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
+    check(
+        load().shk_attention_prefill_bf16(
+            _dev(q, "q"), q.stride(0), _dev(out, "out"), num_tiles, heads, kv_heads, head_dim,
+            _dev(cu_q, "cu_q", torch.int32), _dev(ctx_lens, "ctx_lens", torch.int32),
+            _dev(tile_seq, "tile_seq", torch.int32), _dev(tile_q0, "tile_q0", torch.int32),
+            _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
+            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), _stream(),
         )
     )
 

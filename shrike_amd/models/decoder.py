@@ -53,7 +53,7 @@ class DecoderModel:
         self.embed = tensors[self.embed_name]
         head = tensors.get(self.head_name)
         # shrike/models/qwen.py:211-212: tied and absent -> the embedding table itself
-        self.head = self.embed if head is None else head
+        self.head = runtime.weight(self.embed if head is None else head)
         self.linear = runtime.linear
 
     # ------------------------------------------------------------------ forward

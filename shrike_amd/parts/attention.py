@@ -61,17 +61,17 @@ class PagedAttention(Mixer):
 
     def load(self, tensors, runtime):
         s, n = self.spec, self.name
-        self.w_qkv = torch.cat(
+        self.w_qkv = runtime.weight(torch.cat(
             [tensors[f"{n}.q_proj.weight"], tensors[f"{n}.k_proj.weight"], tensors[f"{n}.v_proj.weight"]],
             dim=0,
-        ).contiguous()
+        ))
         self.b_qkv = (
             torch.cat([tensors[f"{n}.q_proj.bias"], tensors[f"{n}.k_proj.bias"], tensors[f"{n}.v_proj.bias"]])
             .contiguous()
             if s.qkv_bias
             else None
         )
-        self.w_o = tensors[f"{n}.o_proj.weight"].contiguous()
+        self.w_o = runtime.weight(tensors[f"{n}.o_proj.weight"])
         self.b_o = tensors[f"{n}.o_proj.bias"] if s.out_bias else None
         if self.position is not None:
             self.position.load(tensors, runtime)

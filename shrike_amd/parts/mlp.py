@@ -23,10 +23,10 @@ class SwiGLU(FeedForward):
 
     def load(self, tensors, runtime):
         self.inter = int(self.spec.intermediate_size)
-        self.w_gate_up = torch.cat(
+        self.w_gate_up = runtime.weight(torch.cat(
             [tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]], dim=0
-        ).contiguous()
-        self.w_down = tensors[f"{self.name}.down_proj.weight"].contiguous()
+        ))
+        self.w_down = runtime.weight(tensors[f"{self.name}.down_proj.weight"])
         self.linear = runtime.linear
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:

@@ -136,7 +136,7 @@ def paged_setup(seq_lens, page_size, num_pages, kv_heads, head_dim, dtype, seed=
         need = -(-n // page_size)
         tables.append([perm.pop() for _ in range(need)] + [0] * (width - need))
     k_pool = torch.full((num_pages, kv_heads, page_size, head_dim), float("nan"), dtype=dtype, device="cuda")
-    v_pool = torch.full_like(k_pool, float("nan"))
+    v_pool = torch.full((num_pages, kv_heads, head_dim, page_size), float("nan"), dtype=dtype, device="cuda")
     return torch.tensor(tables, dtype=torch.int32, device="cuda"), k_pool, v_pool
 
 
@@ -165,7 +165,7 @@ def test_rope_kv_store(ops, dtype, heads, kv_heads, head_dim, page_size, theta):
         s, p = int(token_seq[t]), int(positions[t])
         page = int(tables[s, p // page_size])
         close(k_pool[page, :, p % page_size], plain.apply_rope(k[t : t + 1], cos[t : t + 1], sin[t : t + 1])[0], dtype)
-        assert torch.equal(v_pool[page, :, p % page_size].cpu().double(), v[t])
+        assert torch.equal(v_pool[page, :, :, p % page_size].cpu().double(), v[t])
     # nothing else was written: every other slot is still NaN
     written = sum(seq_lens) * kv_heads * head_dim
     assert int((~torch.isnan(k_pool.float())).sum()) == written
@@ -181,7 +181,7 @@ def reference_attention(q, k_pool, v_pool, tables, seq_lens, starts, page_size, 
         ctx = start + n_new
         pages = tables[s, : -(-ctx // page_size)].long().cpu()
         k = k_pool.cpu().double()[pages].permute(0, 2, 1, 3).reshape(-1, k_pool.shape[1], k_pool.shape[3])[:ctx]
-        v = v_pool.cpu().double()[pages].permute(0, 2, 1, 3).reshape(-1, v_pool.shape[1], v_pool.shape[3])[:ctx]
+        v = v_pool.cpu().double()[pages].permute(0, 3, 1, 2).reshape(-1, v_pool.shape[1], v_pool.shape[2])[:ctx]
         k, v = torch.nan_to_num(k), torch.nan_to_num(v)  # slots outside the window may be poisoned
         full_q = torch.zeros(ctx, heads, q.shape[2], dtype=torch.float64)
         full_q[start:] = q[off : off + n_new]
@@ -210,7 +210,7 @@ def test_attention_mixed_batch(ops, dtype, heads, kv_heads, head_dim, page_size,
         for p in range(c):
             page = int(tables[s, p // page_size])
             k_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
-            v_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
+            v_pool[page, :, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
     n = sum(seq_lens)
     q = torch.randn(n, heads, head_dim).to(dtype)
     token_seq = torch.cat([torch.full((l,), i) for i, l in enumerate(seq_lens)]).int()
@@ -237,7 +237,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
     for p in range(ctx):
         page = int(tables[0, p // page_size])
         k_pool[page, :, p % page_size] = k[p].to(dtype)
-        v_pool[page, :, p % page_size] = v[p].to(dtype)
+        v_pool[page, :, :, p % page_size] = v[p].to(dtype)
     out = torch.empty(1, heads * head_dim, device="cuda", dtype=dtype)
     ops.attention(dev(q, dtype).view(1, -1), out, heads, kv_heads, head_dim, torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"),
                   torch.zeros(1, dtype=torch.int32, device="cuda"), tables, k_pool, v_pool, page_size, None, 1.0)
@@ -262,7 +262,7 @@ def test_attention_window_edge(ops, dtype):
     for p in range(ctx):
         page = int(tables[0, p // page_size])
         k_pool[page, :, p % page_size] = k[p].to(dtype)
-        v_pool[page, :, p % page_size] = v[p].to(dtype)
+        v_pool[page, :, :, p % page_size] = v[p].to(dtype)
     args = (heads, kv_heads, head_dim, torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"),
             torch.zeros(1, dtype=torch.int32, device="cuda"), tables, k_pool, v_pool, page_size)
     out = torch.empty(1, head_dim, device="cuda", dtype=dtype)
@@ -280,9 +280,10 @@ def test_attention_refuses_head_sizes_it_cannot_do(ops):
 
     with pytest.raises(KernelError, match="head_dim"):
         z = torch.zeros(1, 272, device="cuda")
-        pool = torch.zeros(2, 1, 4, 272, device="cuda")
+        k_pool = torch.zeros(2, 1, 4, 272, device="cuda")
+        v_pool = torch.zeros(2, 1, 272, 4, device="cuda")
         i = torch.zeros(1, dtype=torch.int32, device="cuda")
-        ops.attention(z, torch.empty_like(z), 1, 1, 272, i, i, i.view(1, 1), pool, pool, 4, None, 1.0)
+        ops.attention(z, torch.empty_like(z), 1, 1, 272, i, i, i.view(1, 1), k_pool, v_pool, 4, None, 1.0)
 
 
 # ------------------------------------------------------------------- sampling
@@ -360,3 +361,142 @@ def test_sample_frequencies_follow_the_distribution(ops):
     got = torch.tensor(run_sample(ops, logits, [1.0] * 4096, [1.0] * 4096, us))
     freq = torch.bincount(got, minlength=4).float() / 4096
     assert torch.allclose(freq, probs, atol=0.03)
+
+
+# ------------------------------------------------------ bfloat16 MFMA kernels
+
+
+@pytest.mark.parametrize(
+    "n, m, k",
+    [(1, 48, 64), (8, 3584, 3584), (7, 503, 128), (16, 100, 172), (17, 130, 96), (33, 200, 333),
+     (48, 64, 64), (64, 1000, 520), (5, 37, 50)],
+)
+def test_gemm_tiled_weight(ops, n, m, k):
+    """The weight-streaming MFMA kernel over the tiled weight layout, at sizes
+    that are no multiple of the 16 x 32 tile and rows that are not 16-byte aligned."""
+    torch.manual_seed(12)
+    dtype = torch.bfloat16
+    a, w, b = torch.randn(n, k), torch.randn(m, k) / math.sqrt(k), torch.randn(m)
+    want = rounded(a, dtype) @ rounded(w, dtype).t() + b.double()
+    wt = ops.retile_weight(dev(w, dtype))
+    assert wt.numel() == -(-m // 16) * -(-k // 32) * 512
+    out = torch.empty(n, m, device="cuda", dtype=dtype)
+    ops.gemm_tiled_weight(dev(a, dtype), wt, m, k, out, bias=dev(b))
+    close(out, want, dtype)
+    out32 = torch.full((n, m), 2.0, device="cuda")
+    ops.gemm_tiled_weight(dev(a, dtype), wt, m, k, out32, accumulate=True)
+    close(out32, want - b.double() + 2.0, torch.float32, scale=want.abs().max() * 20)  # float32 sums of bfloat16 products
+    # a strided view of the activations (rows of a wider buffer)
+    wide = torch.zeros(n, k + 24, device="cuda", dtype=dtype)
+    wide[:, :k] = dev(a, dtype)
+    out2 = torch.empty(n, m, device="cuda", dtype=dtype)
+    ops.gemm_tiled_weight(wide[:, :k], wt, m, k, out2, bias=dev(b))
+    assert torch.equal(out2, out)
+
+
+def test_gemm_tiled_weight_rows_do_not_depend_on_the_rest_of_the_batch(ops):
+    torch.manual_seed(13)
+    a, w = dev(torch.randn(40, 256), torch.bfloat16), dev(torch.randn(96, 256), torch.bfloat16)
+    wt = ops.retile_weight(w)
+    full = torch.empty(40, 96, device="cuda")
+    ops.gemm_tiled_weight(a, wt, 96, 256, full)
+    one = torch.empty(1, 96, device="cuda")
+    ops.gemm_tiled_weight(a[23:24], wt, 96, 256, one)
+    assert torch.equal(one[0], full[23])
+
+
+def fill_pools(tables, k_pool, v_pool, ctx, page_size):
+    kv_heads, head_dim = k_pool.shape[1], k_pool.shape[3]
+    for s, c in enumerate(ctx):
+        for p in range(c):
+            page = int(tables[s, p // page_size])
+            k_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(k_pool.dtype)
+            v_pool[page, :, :, p % page_size] = torch.randn(kv_heads, head_dim).to(v_pool.dtype)
+
+
+@pytest.mark.parametrize(
+    "heads, kv_heads, head_dim, page_size, window, nsplit",
+    [(14, 2, 64, 16, None, 1), (14, 2, 64, 16, None, 5), (28, 4, 128, 16, None, 8), (6, 3, 96, 32, 40, 3),
+     (16, 1, 32, 64, None, 2), (5, 5, 256, 16, 100, 4), (8, 8, 160, 48, None, 64)],
+)
+def test_attention_decode_mfma(ops, heads, kv_heads, head_dim, page_size, window, nsplit):
+    """Context lengths of the reference's decode test (tests/test_triton_attention.py:40-42),
+    distinct random pages, unused slots poisoned with NaN."""
+    torch.manual_seed(14)
+    dtype = torch.bfloat16
+    assert ops.attention_supports_mfma(heads, kv_heads, head_dim, page_size, heads * head_dim)
+    ctx = [1, 15, 16, 17, 100, 333, 512, 7, 31, 32, 33, 129]
+    n = len(ctx)
+    num_pages = sum(-(-c // page_size) for c in ctx) + 5
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, num_pages, kv_heads, head_dim, dtype, seed=2)
+    fill_pools(tables, k_pool, v_pool, ctx, page_size)
+    q = torch.randn(n, heads, head_dim).to(dtype)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32)
+    out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
+    partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
+    scale = 1.3 * head_dim**-0.5
+    ops.attention_decode(dev(q).view(n, -1), out, n, heads, kv_heads, head_dim, dev(positions), tables,
+                         k_pool, v_pool, page_size, window, scale, partial, nsplit)
+    want = reference_attention(q.double(), k_pool, v_pool, tables, [1] * n, [c - 1 for c in ctx], page_size, window, scale)
+    assert not torch.isnan(out.float()).any(), "a slot outside the context reached the output"
+    close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
+
+
+@pytest.mark.parametrize(
+    "heads, kv_heads, head_dim, page_size, window",
+    [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 256, 16, None)],
+)
+def test_attention_prefill_mfma(ops, heads, kv_heads, head_dim, page_size, window):
+    """Portions of 2 to 200 tokens, some with earlier context, tiles with fewer than 16 queries."""
+    torch.manual_seed(15)
+    dtype = torch.bfloat16
+    seq_lens = [2, 200, 16, 17, 90, 33]
+    starts = [0, 60, 5, 100, 0, 31]
+    ctx = [s + l for s, l in zip(starts, seq_lens)]
+    n = sum(seq_lens)
+    num_pages = sum(-(-c // page_size) for c in ctx) + 5
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, num_pages, kv_heads, head_dim, dtype, seed=3)
+    fill_pools(tables, k_pool, v_pool, ctx, page_size)
+    q = torch.randn(n, heads, head_dim).to(dtype)
+    cu = [0]
+    for l in seq_lens:
+        cu.append(cu[-1] + l)
+    tile_seq, tile_q0 = [], []
+    for s, l in enumerate(seq_lens):
+        for q0 in range(0, l, 16):
+            tile_seq.append(s)
+            tile_q0.append(q0)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
+    scale = head_dim**-0.5
+    ops.attention_prefill(dev(q).view(n, -1), out, len(tile_seq), heads, kv_heads, head_dim, i32(cu), i32(ctx),
+                          i32(tile_seq), i32(tile_q0), tables, k_pool, v_pool, page_size, window, scale)
+    want = reference_attention(q.double(), k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale)
+    assert not torch.isnan(out.float()).any()
+    close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
+
+
+def test_attention_mfma_finds_one_far_key_among_thousands(ops):
+    """Decode over 3000 keys split 16 ways: one key in an early page is made to stand out."""
+    torch.manual_seed(16)
+    dtype = torch.bfloat16
+    heads, kv_heads, head_dim, page_size, ctx = 14, 2, 128, 16, 3000
+    tables, k_pool, v_pool = paged_setup([ctx], page_size, 256, kv_heads, head_dim, dtype, seed=4)
+    k = torch.randn(ctx, kv_heads, head_dim) * 0.1
+    v = torch.randn(ctx, kv_heads, head_dim)
+    q = torch.randn(1, heads, head_dim)
+    far = 41
+    k[far, 0] = q[0, 3] * 2.0  # head 3 of group 0
+    for p in range(ctx):
+        page = int(tables[0, p // page_size])
+        k_pool[page, :, p % page_size] = k[p].to(dtype)
+        v_pool[page, :, :, p % page_size] = v[p].to(dtype)
+    out = torch.empty(1, heads * head_dim, device="cuda", dtype=dtype)
+    partial = torch.empty(heads * 16 * (head_dim + 2), device="cuda")
+    ops.attention_decode(dev(q, dtype).view(1, -1), out, 1, heads, kv_heads, head_dim,
+                         torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"), tables, k_pool, v_pool,
+                         page_size, None, 1.0, partial, 16)
+    got = out.view(heads, head_dim).float().cpu()
+    assert torch.allclose(got[3], v[far, 0].to(dtype).float(), atol=3e-2)
+    want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, [1], [ctx - 1], page_size, None, 1.0)
+    close(out.view(1, heads, head_dim), want, dtype, scale=1.0)
