@@ -1,0 +1,246 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+The model has the layer sizes of the Qwen2.5-7B shape (BASELINE.json
+configs[2]) with random weights in bfloat16.  A "step" is one decode step of
+the whole serving path (LLMEngine.step: schedule, forward from the paged cache,
+sample, book-keeping) for `batch` requests that were each prefilled with 2,048
+random tokens; decoding runs towards context 4,096.  One JSON line is printed:
+`value` is decoded tokens per second; `prefill` is a 2,048-token prompt in one
+step; `roofline` prices the decode step's unavoidable HBM reads (every weight
+once, the live requests' cache) against 8 TB/s; `points` holds batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import random
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# Qwen2.5-7B shape: BASELINE.json configs[2]
+SHAPE_7B = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "hidden_size": 3584,
+    "intermediate_size": 18944,
+    "num_hidden_layers": 28,
+    "num_attention_heads": 28,
+    "num_key_value_heads": 4,
+    "head_dim": 128,
+    "vocab_size": 152064,
+    "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False,
+    "attention_bias": True,
+    "max_position_embeddings": 32768,
+    "eos_token_id": 151645,
+    "torch_dtype": "bfloat16",
+}
+PROMPT_LEN = 2048
+CONTEXT_END = 4096
+PAGE_SIZE = 16
+HBM_PEAK_GBS = 8000.0
+BF16_PEAK_FLOPS = 2.5e15
+
+
+def matmul_params(cfg) -> tuple[int, int]:
+    """(elements of all per-layer matrices, elements of the output matrix)."""
+    h, d = cfg.hidden_size, cfg.head_dim
+    per_layer = (
+        (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * d * h
+        + cfg.num_attention_heads * d * h
+        + 3 * h * cfg.intermediate_size
+    )
+    return per_layer * cfg.num_hidden_layers, cfg.vocab_size * h
+
+
+def kv_bytes_per_token(cfg) -> int:
+    return cfg.num_hidden_layers * 2 * cfg.num_key_value_heads * cfg.head_dim * 2
+
+
+def prefill_flops(cfg, n: int) -> float:
+    layers, head = matmul_params(cfg)
+    linear = 2.0 * n * layers + 2.0 * head  # the output matrix runs on one row
+    # causal attention: token p reads p + 1 keys, 2 products of head_dim each per head
+    attn = 4.0 * cfg.head_dim * cfg.num_attention_heads * cfg.num_hidden_layers * n * (n + 1) / 2
+    return linear + attn
+
+
+def make_engine(cfg, spec, max_batch: int, seed: int):
+    import torch
+
+    from shrike_amd.config import EngineConfig
+    from shrike_amd.engine.llm_engine import LLMEngine
+    from shrike_amd.engine.loading import random_model
+
+    t0 = time.perf_counter()
+    model, runtime = random_model(spec, seed=seed, dtype="bfloat16")
+    torch.cuda.synchronize()
+    print(f"[bench] random weights on the device in {time.perf_counter() - t0:.1f}s", file=sys.stderr)
+    pages = max_batch * (CONTEXT_END // PAGE_SIZE + 2)
+    config = EngineConfig(
+        block_size=PAGE_SIZE, num_kv_blocks=pages, max_tokens_per_step=PROMPT_LEN + max_batch,
+        max_running=max_batch, enable_prefix_caching=False, dtype="bfloat16", seed=seed,
+    )
+    return LLMEngine(None, config, model=model, runtime=runtime)
+
+
+def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int) -> dict:
+    """Prefill `batch` prompts, then time `steps` decode steps."""
+    import torch
+
+    from shrike_amd import SamplingParams
+
+    rng = random.Random(seed)
+    sampling = SamplingParams(max_new_tokens=batch + warmup + steps + 8, ignore_eos=True)
+    for _ in range(batch):
+        engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)], sampling)
+    while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
+        engine.step()
+    for _ in range(warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    context_start = sum(r.num_computed_tokens for r in engine.scheduler.running) / batch
+    t0 = time.perf_counter()
+    produced = 0
+    for _ in range(steps):
+        produced += len(engine.step())
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    context_end = sum(r.num_computed_tokens for r in engine.scheduler.running) / batch
+    assert produced == batch * steps, f"{produced} tokens from {steps} steps of {batch}"
+    for req in list(engine.scheduler.running):
+        engine.abort(req.req_id)
+    layer_w, head_w = matmul_params(cfg)
+    mean_ctx = (context_start + context_end) / 2 + 1
+    step_bytes = 2.0 * (layer_w + head_w) + batch * mean_ctx * kv_bytes_per_token(cfg)
+    ms = elapsed / steps * 1e3
+    return {
+        "tok_s": produced / elapsed, "ms_per_step": ms, "context_start": context_start,
+        "context_end": context_end, "step_bytes": step_bytes,
+        "gb_s": step_bytes / (ms * 1e-3) / 1e9,
+    }
+
+
+def run_prefill(engine, cfg, seed: int, repeats: int = 3) -> dict:
+    import torch
+
+    from shrike_amd import SamplingParams
+
+    rng = random.Random(seed + 1)
+    best = None
+    for _ in range(repeats):
+        engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)],
+                           SamplingParams(max_new_tokens=1, ignore_eos=True))
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        outs = engine.step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert len(outs) == 1 and outs[0].finished
+        best = dt if best is None else min(best, dt)
+    flops = prefill_flops(cfg, PROMPT_LEN)
+    return {"value": round(PROMPT_LEN / best, 1), "tokens": PROMPT_LEN, "ms": round(best * 1e3, 3),
+            "frac": round(flops / best / BF16_PEAK_FLOPS, 4)}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
+    ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
+    ap.add_argument("--steps", type=int, default=2048 - 8)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=SHAPE_7B["num_hidden_layers"],
+                    help="run fewer layers than the configuration has (both numbers are reported)")
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    if args.steps < 1 or args.warmup < 0 or args.batch < 1:
+        print("bench.py: --steps and --batch must be positive, --warmup non-negative")
+        return 2
+    room = CONTEXT_END - PROMPT_LEN - args.warmup - max(args.batch, 1 if args.no_points else 64) - 2
+    if args.steps > room:
+        print(f"bench.py: at most {room} steps fit between the prompt and context {CONTEXT_END}")
+        return 2
+
+    import torch
+
+    import shrike_amd.models  # noqa: F401
+    from shrike_amd.models.qwen2 import Qwen2Config, build_spec
+
+    raw = dict(SHAPE_7B, num_hidden_layers=args.layers)
+    cfg = Qwen2Config.from_dict(raw)
+    spec = build_spec(cfg)
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    engine = make_engine(cfg, spec, max(batches), args.seed)
+
+    results = {}
+    for b in batches:
+        results[b] = run_decode(engine, cfg, b, args.steps, args.warmup, args.seed + b)
+        print(f"[bench] batch {b}: {results[b]['tok_s']:.1f} tok/s, "
+              f"{results[b]['ms_per_step']:.3f} ms/step, {results[b]['gb_s']:.0f} GB/s",
+              file=sys.stderr)
+    prefill = run_prefill(engine, cfg, args.seed)
+    print(f"[bench] prefill: {prefill}", file=sys.stderr)
+
+    main_run = results[args.batch]
+    line = {
+        "metric": "decode tok/s at batch 8 (Qwen2.5-7B shape, 2048-token prompts, decode to 4096)",
+        "value": round(main_run["tok_s"], 1),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic: random weights N(0, 0.02), prompt ids uniform in [0, vocab)",
+        "config": {
+            "model": "Qwen2.5-7B shape (Qwen2ForCausalLM)",
+            "layers": cfg.num_hidden_layers,
+            "layers_of_config": SHAPE_7B["num_hidden_layers"],
+            "hidden": cfg.hidden_size,
+            "heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim,
+            "intermediate": cfg.intermediate_size,
+            "vocab": cfg.vocab_size,
+            "global_batch": args.batch,
+            "seq_len": CONTEXT_END,
+            "prompt_len": PROMPT_LEN,
+            "context_start": round(main_run["context_start"], 1),
+            "context_end": round(main_run["context_end"], 1),
+            "page_size": PAGE_SIZE,
+            "parallelism": "single GPU",
+            "sampling": "greedy",
+            "hip_graphs": True,
+        },
+        "prefill": prefill,
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(main_run["gb_s"], 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(main_run["gb_s"] / HBM_PEAK_GBS, 4),
+        },
+        "points": {f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
+    }
+    line["points"][f"decode_b{args.batch}"] = round(main_run["tok_s"], 1)
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

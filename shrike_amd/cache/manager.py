@@ -124,12 +124,14 @@ class CacheManager:
 
         for g in self.groups:
             s = g.spec
+            # one page more than the pool hands out: page `num_pages` is where the
+            # padding rows of a fixed-size (graph) batch put their keys and values
             g.k_tensor = torch.zeros(
-                len(g.layers), self.num_pages, s.num_kv_heads, self.page_size, s.head_dim,
+                len(g.layers), self.num_pages + 1, s.num_kv_heads, self.page_size, s.head_dim,
                 dtype=dtype, device=device,
             )
             g.v_tensor = torch.zeros(
-                len(g.layers), self.num_pages, s.num_kv_heads, s.head_dim, self.page_size,
+                len(g.layers), self.num_pages + 1, s.num_kv_heads, s.head_dim, self.page_size,
                 dtype=dtype, device=device,
             )
         for g in self.state_groups:

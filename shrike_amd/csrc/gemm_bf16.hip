@@ -122,6 +122,127 @@ __global__ void __launch_bounds__(kSkinnyWaves* kWave)
   }
 }
 
+// gemm_big_kernel: for many tokens (prompt portions).  A workgroup of 4
+// wavefronts computes 128 weight rows x 128 tokens; each wavefront a 64 x 64
+// quadrant as 4 x 4 MFMA tiles.  Per stage of 64 columns of k, the weights'
+// tiles (already in operand layout) and the activations (re-laid on the way)
+// are staged in LDS "fragment-major": the 16 bytes of lane l of a fragment sit
+// at l * 16, so every LDS access is a conflict-free 128-bit access.  Stages are
+// double-buffered: the loads of stage t+1 are in flight while stage t is
+// multiplied.
+
+constexpr int kBigM = 128;   // weight rows per workgroup
+constexpr int kBigN = 128;   // tokens per workgroup
+constexpr int kBigK = 64;    // k per stage (two MFMA steps)
+constexpr int kBigFrags = (kBigM / 16) * (kBigK / 32);  // fragments per operand per stage: 16
+
+__global__ void __launch_bounds__(256)
+    gemm_big_kernel(const bf16* __restrict__ a, int lda, int n, int k,
+                    const uint4* __restrict__ wt, int ktiles, int m,
+                    const float* __restrict__ bias, void* __restrict__ out, int ldo, int out_f32,
+                    int accumulate, int vec) {
+  // [buffer][operand: 0 weights, 1 activations][fragment][lane]
+  __shared__ uint4 stage[2][2][kBigFrags][kWave];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave / 2, wn = wave % 2;  // quadrant of the wavefront
+  const int mb0 = blockIdx.x * (kBigM / 16);   // first block of 16 weight rows
+  const int tok0 = blockIdx.y * kBigN;
+  const int mblocks = (m + 15) / 16;
+  const int nstages = (ktiles + 1) / 2;
+
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int jn = 0; jn < 4; ++jn) acc[i][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // Each thread moves 4 fragments-lanes per operand per stage: fragment f = tid/64 + 4*i
+  // (f = rb * 2 + ks: block of 16 rows rb, MFMA step ks), lane = tid % 64.
+  uint4 wreg[4], areg[4];
+  auto load_stage = [&](int st) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int f = wave + 4 * i, rb = f / 2, ks = f % 2;
+      const int kt = st * 2 + ks;
+      const int mb = mb0 + rb;
+      wreg[i] = make_uint4(0, 0, 0, 0);
+      if (mb < mblocks && kt < ktiles)
+        wreg[i] = wt[(static_cast<size_t>(mb) * ktiles + kt) * kWave + lane];
+      const int token = tok0 + rb * 16 + lane % 16;
+      areg[i] = load_act(a, lda, n, k, token, kt * 32 + (lane / 16) * 8, vec).u;
+    }
+  };
+  auto store_stage = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int f = wave + 4 * i;
+      stage[buf][0][f][lane] = wreg[i];
+      stage[buf][1][f][lane] = areg[i];
+    }
+  };
+
+  load_stage(0);
+  store_stage(0);
+  __syncthreads();
+  for (int st = 0; st < nstages; ++st) {
+    const int buf = st & 1;
+    if (st + 1 < nstages) load_stage(st + 1);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      Frag wf[4], af[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) wf[i].u = stage[buf][0][(wm * 4 + i) * 2 + ks][lane];
+#pragma unroll
+      for (int jn = 0; jn < 4; ++jn) af[jn].u = stage[buf][1][(wn * 4 + jn) * 2 + ks][lane];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int jn = 0; jn < 4; ++jn)
+          acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, af[jn].v, acc[i][jn], 0, 0, 0);
+    }
+    if (st + 1 < nstages) store_stage(buf ^ 1);
+    __syncthreads();
+  }
+
+  // lane (j, kg) of tile (i, jn): token tok0 + (wn*4 + jn)*16 + j, rows (mb0 + wm*4 + i)*16 + kg*4 + r
+  const int j = lane % 16, kg = lane / 16;
+#pragma unroll
+  for (int jn = 0; jn < 4; ++jn) {
+    const int token = tok0 + (wn * 4 + jn) * 16 + j;
+    if (token >= n) continue;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row0 = (mb0 + wm * 4 + i) * 16 + kg * 4;
+      if (row0 >= m) continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = acc[i][jn][r];
+        if (bias && row0 + r < m) v[r] += bias[row0 + r];
+      }
+      const size_t idx = static_cast<size_t>(token) * ldo + row0;
+      if (out_f32) {
+        float* o = static_cast<float*>(out) + idx;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+      } else {
+        bf16* o = static_cast<bf16*>(out) + idx;
+        if (row0 + 3 < m && (ldo & 3) == 0) {
+          uint2 packed;
+          packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+          packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+          *reinterpret_cast<uint2*>(o) = packed;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (row0 + r < m) o[r] = from_float<bf16>(v[r]);
+        }
+      }
+    }
+  }
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -160,7 +281,6 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   SHK_REQUIRE(n >= 0 && m > 0 && k > 0, "gemm_bf16: bad sizes n=%d m=%d k=%d", n, m, k);
   SHK_REQUIRE(lda >= k && ldo >= m, "gemm_bf16: row strides lda=%d ldo=%d too small", lda, ldo);
   SHK_REQUIRE(!accumulate || out_dtype == kF32, "gemm_bf16: accumulate needs a float32 output");
-  SHK_REQUIRE(n <= 64, "gemm_bf16: the skinny kernel takes at most 64 rows, got %d", n);
   if (n == 0) return 0;
   SHK_REQUIRE(a && wt && out, "gemm_bf16: null pointer");
   const int mb = (m + 15) / 16, kt = (k + 31) / 32;
@@ -169,6 +289,15 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   const bf16* ap = static_cast<const bf16*>(a);
   const uint4* wp = static_cast<const uint4*>(wt);
   const int of = out_dtype == kF32;
+  if (n > 64) {
+    SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
+    dim3 grid((m + kBigM - 1) / kBigM, (n + kBigN - 1) / kBigN);
+    SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);
+    gemm_big_kernel<<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate,
+                                         vec);
+    SHK_LAUNCH_CHECK("gemm_bf16");
+    return 0;
+  }
 #define SHK_SKINNY(NB)                                                                        \
   gemm_skinny_kernel<NB><<<mb, kSkinnyWaves * kWave, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, \
                                                              out, ldo, of, accumulate, vec)

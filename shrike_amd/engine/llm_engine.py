@@ -64,7 +64,7 @@ class LLMEngine:
         self.cache = CacheManager(specs, cfg.block_size, num_blocks, max_slots=cfg.max_running,
                                   enable_prefix_caching=cfg.enable_prefix_caching)
         self.cache.allocate(runtime.dtype, runtime.device)
-        self.runner = ModelRunner(model, self.cache, runtime)
+        self.runner = ModelRunner(model, self.cache, runtime, graphs=cfg.graphs)
         self.scheduler = Scheduler(self.cache, cfg.max_tokens_per_step, cfg.max_running)
         self.sampler = Sampler(runtime.device, cfg.seed)
         self.eos_ids = set(model.spec.eos_token_ids)

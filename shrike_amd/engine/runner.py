@@ -4,8 +4,10 @@ for the wanted places only.
 
 Reference: shrike/engine/model_runner.py:183-250.  Differences by design: the
 entries carry their tokens and wanted rows explicitly (so replay can ask for
-any row), all metadata goes to the device in one copy, and nothing is computed
-on the host per token.
+any row), all metadata goes to the device in one copy, nothing is computed on
+the host per token, and steps that hold only single tokens are replayed from
+HIP graphs (one per batch-size bucket), because such a step is a few hundred
+short kernels whose launches would otherwise cost more than they run.
 """
 
 from __future__ import annotations
@@ -17,6 +19,10 @@ import torch
 
 from ..cache.manager import CacheManager, SequenceCache
 from .context import StepContext, Workspace
+from .runtime import bucket
+
+GRAPH_BATCH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
+GRAPH_TABLE_QUANTUM = 64  # block-table widths of graphs are multiples of this
 
 
 @dataclass
@@ -34,8 +40,45 @@ class StepError(ValueError):
     """A step was refused before anything ran."""
 
 
+class _Meta:
+    """The int32 metadata of a step, laid out in one buffer."""
+
+    FIELDS = ("token_ids", "positions", "token_seq", "cu_q", "ctx_lens", "state_slots", "fresh",
+              "out_rows", "tile_seq", "tile_q0")
+
+    def __init__(self, arrays: dict, tables: list[np.ndarray]):
+        self.arrays = arrays
+        self.tables = tables
+        self.parts = [arrays[f] for f in self.FIELDS] + [t.reshape(-1) for t in tables]
+        self.sizes = [int(p.size) for p in self.parts]
+        self.total = int(sum(self.sizes))
+
+    def views(self, dev: torch.Tensor, num_seqs: int) -> dict:
+        out, off = {}, 0
+        for name, size in zip(self.FIELDS, self.sizes):
+            out[name] = dev[off : off + size]
+            off += size
+        tables = []
+        for t in self.tables:
+            tables.append(dev[off : off + t.size].view(num_seqs, t.shape[1]))
+            off += t.size
+        out["block_tables"] = tables
+        return out
+
+
+class _DecodeGraph:
+    """A captured decode step for one (batch bucket, table widths, context bucket)."""
+
+    def __init__(self, device):
+        self.workspace = Workspace(device)
+        self.graph = None
+        self.meta_dev = None
+        self.logits = None
+        self.ctx = None
+
+
 class ModelRunner:
-    def __init__(self, model, cache: CacheManager, runtime):
+    def __init__(self, model, cache: CacheManager, runtime, graphs: bool = True):
         self.model = model
         self.cache = cache
         self.runtime = runtime
@@ -50,6 +93,11 @@ class ModelRunner:
                 self.layer_caches.append(None)
         self._pinned = None
         self._pinned_free = None  # event: the last copy out of the pinned buffer is done
+        # Graphs replay fixed kernel arguments: a mixer that reads host-side
+        # metadata (state kept outside the kernels' view) cannot be captured.
+        self.use_graphs = bool(graphs) and not cache.state_groups
+        self._graphs: dict[tuple, _DecodeGraph] = {}
+        self.graph_replays = 0
 
     # ---------------------------------------------------------------- metadata
 
@@ -78,83 +126,161 @@ class ModelRunner:
                 if any(p < 0 or p >= self.cache.num_pages for p in table[first : last_page + 1]):
                     raise StepError("block table names a page outside the pool")
 
-    def build_context(self, entries: list[StepEntry]) -> StepContext:
-        self._check(entries)
-        order = sorted(range(len(entries)), key=lambda i: 0 if len(entries[i].tokens) == 1 else 1)
+    def _meta(self, entries: list[StepEntry], order: list[int], pad_to: int = 0,
+              table_widths: list[int] | None = None) -> _Meta:
+        """Arrays of the step.  With pad_to, rows are added up to that many
+        sequences: one token each at position 0 whose page is the spare page
+        that no request ever holds."""
+        n_real = len(order)
         q_lens = np.array([len(entries[i].tokens) for i in order], dtype=np.int64)
         starts = np.array([entries[i].start for i in order], dtype=np.int64)
-        num_seqs = len(order)
+        pads = max(0, pad_to - n_real)
+        if pads:
+            q_lens = np.concatenate([q_lens, np.ones(pads, dtype=np.int64)])
+            starts = np.concatenate([starts, np.zeros(pads, dtype=np.int64)])
+        num_seqs = n_real + pads
         num_tokens = int(q_lens.sum())
         num_decode = int((q_lens == 1).sum())
         cu_q = np.zeros(num_seqs + 1, dtype=np.int64)
         np.cumsum(q_lens, out=cu_q[1:])
         token_seq = np.repeat(np.arange(num_seqs), q_lens)
         positions = np.arange(num_tokens) - cu_q[token_seq] + starts[token_seq]
-        token_ids = np.concatenate([np.asarray(entries[i].tokens, dtype=np.int64) for i in order])
+        token_ids = np.concatenate(
+            [np.asarray(entries[i].tokens, dtype=np.int64) for i in order]
+            + [np.zeros(pads, dtype=np.int64)]
+        )
         if token_ids.min() < 0 or token_ids.max() >= self.vocab_size:
             raise StepError(f"token ids must lie in [0, {self.vocab_size})")
         ctx_lens = starts + q_lens
         slot_of = {i: k for k, i in enumerate(order)}
-        out_rows = [cu_q[slot_of[i]] + w for i, e in enumerate(entries) for w in e.want]
-        state_slots = np.array([entries[i].cache.state_slot for i in order], dtype=np.int64)
-        fresh = np.array([int(entries[i].cache.fresh_state) for i in order], dtype=np.int64)
+        if pad_to:
+            out_rows = np.arange(num_seqs, dtype=np.int64)  # one row per sequence, pads included
+        else:
+            out_rows = np.asarray(
+                [cu_q[slot_of[i]] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int64
+            )
+        state_slots = np.array([entries[i].cache.state_slot for i in order] + [0] * pads,
+                               dtype=np.int64)
+        fresh = np.array([int(entries[i].cache.fresh_state) for i in order] + [0] * pads,
+                         dtype=np.int64)
         tables = []
         for gi in range(len(self.cache.groups)):
-            width = max(1, max(len(entries[i].cache.tables[gi]) for i in order))
+            need = max(1, max(len(entries[i].cache.tables[gi]) for i in order))
+            width = table_widths[gi] if table_widths else need
             t = np.zeros((num_seqs, width), dtype=np.int64)
             for k, i in enumerate(order):
                 row = entries[i].cache.tables[gi]
                 t[k, : len(row)] = row
+            t[n_real:, :] = self.cache.num_pages  # the spare page
             tables.append(t)
-
         # prompt portions in tiles of 16 queries for the MFMA attention kernel
         tile_counts = -(-q_lens[num_decode:] // 16)
         tile_seq = np.repeat(np.arange(num_decode, num_seqs), tile_counts)
         tile_first = np.zeros(num_seqs - num_decode + 1, dtype=np.int64)
         np.cumsum(tile_counts, out=tile_first[1:])
         tile_q0 = (np.arange(int(tile_counts.sum())) - tile_first[tile_seq - num_decode]) * 16
+        arrays = dict(token_ids=token_ids, positions=positions, token_seq=token_seq, cu_q=cu_q,
+                      ctx_lens=ctx_lens, state_slots=state_slots, fresh=fresh, out_rows=out_rows,
+                      tile_seq=tile_seq, tile_q0=tile_q0)
+        meta = _Meta(arrays, tables)
+        meta.q_lens, meta.ctx_lens = q_lens, ctx_lens
+        meta.num_seqs, meta.num_tokens, meta.num_decode = num_seqs, num_tokens, num_decode
+        return meta
 
-        parts = [token_ids, positions, token_seq, cu_q, ctx_lens, state_slots, fresh,
-                 np.asarray(out_rows, dtype=np.int64), tile_seq, tile_q0]
-        parts += [t.reshape(-1) for t in tables]
-        sizes = [p.size for p in parts]
-        total = int(sum(sizes))
+    def _upload(self, meta: _Meta, dev: torch.Tensor) -> None:
         if self._pinned_free is not None:
             self._pinned_free.synchronize()
-        if self._pinned is None or self._pinned.numel() < total:
-            self._pinned = torch.empty(max(2 * total, 4096), dtype=torch.int32, pin_memory=True)
+        if self._pinned is None or self._pinned.numel() < meta.total:
+            self._pinned = torch.empty(max(2 * meta.total, 4096), dtype=torch.int32, pin_memory=True)
             self._pinned_free = torch.cuda.Event()
-        host = self._pinned[:total]
-        host.numpy()[:] = np.concatenate(parts).astype(np.int32)
-        dev = self.workspace.get("step_meta", (total,), torch.int32)
+        host = self._pinned[: meta.total]
+        np.concatenate(meta.parts, out=host.numpy(), casting="unsafe")
         dev.copy_(host, non_blocking=True)
         self._pinned_free.record()
-        views, off = [], 0
-        for s in sizes:
-            views.append(dev[off : off + s])
-            off += s
+
+    def _context(self, meta: _Meta, dev: torch.Tensor, workspace: Workspace,
+                 max_decode_ctx: int | None = None) -> StepContext:
+        v = meta.views(dev, meta.num_seqs)
+        nd = meta.num_decode
         return StepContext(
-            dtype=self.runtime.dtype, device=self.runtime.device, workspace=self.workspace,
-            num_tokens=num_tokens, num_seqs=num_seqs, num_decode=num_decode,
-            token_ids=views[0], positions=views[1], token_seq=views[2], cu_q=views[3],
-            ctx_lens=views[4], state_slots=views[5], fresh=views[6], out_rows=views[7],
-            tile_seq=views[8], tile_q0=views[9], num_prefill_tiles=int(tile_seq.size),
-            block_tables=[v.view(num_seqs, t.shape[1]) for v, t in zip(views[10:], tables)],
-            q_lens=q_lens.tolist(), ctx_lens_host=ctx_lens.tolist(),
-            max_q_len=int(q_lens.max()), max_ctx_len=int(ctx_lens.max()),
-            max_decode_ctx=int(ctx_lens[:num_decode].max()) if num_decode else 0,
+            dtype=self.runtime.dtype, device=self.runtime.device, workspace=workspace,
+            num_tokens=meta.num_tokens, num_seqs=meta.num_seqs, num_decode=nd,
+            token_ids=v["token_ids"], positions=v["positions"], token_seq=v["token_seq"],
+            cu_q=v["cu_q"], ctx_lens=v["ctx_lens"], state_slots=v["state_slots"], fresh=v["fresh"],
+            out_rows=v["out_rows"], tile_seq=v["tile_seq"], tile_q0=v["tile_q0"],
+            num_prefill_tiles=int(meta.arrays["tile_seq"].size), block_tables=v["block_tables"],
+            q_lens=meta.q_lens.tolist(), ctx_lens_host=meta.ctx_lens.tolist(),
+            max_q_len=int(meta.q_lens.max()), max_ctx_len=int(meta.ctx_lens.max()),
+            max_decode_ctx=(
+                max_decode_ctx if max_decode_ctx is not None
+                else (int(meta.ctx_lens[:nd].max()) if nd else 0)
+            ),
         )
+
+    def build_context(self, entries: list[StepEntry]) -> StepContext:
+        self._check(entries)
+        order = sorted(range(len(entries)), key=lambda i: 0 if len(entries[i].tokens) == 1 else 1)
+        meta = self._meta(entries, order)
+        dev = self.workspace.get("step_meta", (meta.total,), torch.int32)
+        self._upload(meta, dev)
+        return self._context(meta, dev, self.workspace)
+
+    # ------------------------------------------------------------------ graphs
+
+    def _graph_key(self, entries: list[StepEntry]):
+        """Bucket of a step that holds only single tokens which all want their
+        logits, or None when the step does not qualify."""
+        if not self.use_graphs or len(entries) > GRAPH_BATCH_BUCKETS[-1]:
+            return None
+        for e in entries:
+            if len(e.tokens) != 1 or list(e.want) != [0]:
+                return None
+        batch = next(b for b in GRAPH_BATCH_BUCKETS if b >= len(entries))
+        widths = []
+        for gi in range(len(self.cache.groups)):
+            need = max(len(e.cache.tables[gi]) for e in entries)
+            widths.append(-(-need // GRAPH_TABLE_QUANTUM) * GRAPH_TABLE_QUANTUM)
+        ctx_bucket = bucket(max(e.start + 1 for e in entries), 256)
+        return batch, tuple(widths), ctx_bucket
+
+    def _graph_step(self, entries: list[StepEntry], key) -> torch.Tensor:
+        batch, widths, ctx_bucket = key
+        self._check(entries)
+        order = list(range(len(entries)))
+        meta = self._meta(entries, order, pad_to=batch, table_widths=list(widths))
+        g = self._graphs.get(key)
+        if g is None:
+            g = _DecodeGraph(self.runtime.device)
+            g.meta_dev = torch.zeros(meta.total, dtype=torch.int32, device=self.runtime.device)
+            self._upload(meta, g.meta_dev)
+            g.ctx = self._context(meta, g.meta_dev, g.workspace, max_decode_ctx=ctx_bucket)
+            # once eagerly: every workspace buffer exists before the capture starts
+            self.model.forward(g.ctx, self.layer_caches)
+            torch.cuda.synchronize(self.runtime.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                g.logits = self.model.forward(g.ctx, self.layer_caches)
+            g.graph = graph
+            self._graphs[key] = g
+        self._upload(meta, g.meta_dev)
+        g.graph.replay()
+        self.graph_replays += 1
+        return g.logits[: len(entries)]
 
     # -------------------------------------------------------------------- step
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor:
         """Runs the entries' tokens as one batch; returns float32 logits
         [wanted, vocab] in the order of the entries and of their `want`.
-        The tensor is a view of a buffer that the next step overwrites."""
+        The tensor is a view of a buffer that a later step overwrites."""
         if not entries:
             return torch.empty(0, self.vocab_size, dtype=torch.float32, device=self.runtime.device)
-        ctx = self.build_context(entries)
-        logits = self.model.forward(ctx, self.layer_caches)
+        key = self._graph_key(entries)
+        if key is not None:
+            logits = self._graph_step(entries, key)
+        else:
+            ctx = self.build_context(entries)
+            logits = self.model.forward(ctx, self.layer_caches)
         for e in entries:
             e.cache.fresh_state = False
         return logits

@@ -3,9 +3,10 @@ held, and the choice of kernel for each matrix product and attention call.
 
 float32: every product runs in the general float32 kernel (fused multiply-add,
 no matrix mode of reduced precision) and attention in the general kernel.
-bfloat16: weights are also held in the MFMA operand layout; products with at
-most 64 rows stream them once through the skinny MFMA kernel; attention runs
-on the MFMA kernels where the shapes allow, else in the general kernel.
+bfloat16: weights are held in the MFMA operand layout; products with at most
+64 rows stream them once through the skinny MFMA kernel, larger ones run the
+LDS-staged MFMA kernel; attention runs on the MFMA kernels where the shapes
+allow, else in the general kernel.
 """
 
 from __future__ import annotations
@@ -14,18 +15,15 @@ import torch
 
 from ..kernels import ops
 
-SKINNY_ROWS = 64  # most rows of a step that the weight-streaming kernel takes
-
-
 class LinearWeight:
     """A weight matrix [rows, cols] as the kernels want it."""
 
     __slots__ = ("rows", "cols", "dense", "tiled")
 
-    def __init__(self, dense: torch.Tensor, tiled: torch.Tensor | None):
-        self.rows, self.cols = dense.shape
-        self.dense = dense
-        self.tiled = tiled
+    def __init__(self, shape, dense: torch.Tensor | None, tiled: torch.Tensor | None):
+        self.rows, self.cols = shape
+        self.dense = dense  # row-major (float32 path)
+        self.tiled = tiled  # MFMA operand layout (bfloat16 path)
 
 
 class Runtime:
@@ -38,12 +36,13 @@ class Runtime:
     def weight(self, w: torch.Tensor) -> LinearWeight:
         """Takes a row-major [out, in] matrix in the compute dtype."""
         w = w.contiguous()
-        tiled = ops.retile_weight(w) if self.dtype == torch.bfloat16 else None
-        return LinearWeight(w, tiled)
+        if self.dtype == torch.bfloat16:
+            return LinearWeight(w.shape, None, ops.retile_weight(w))
+        return LinearWeight(w.shape, w, None)
 
     def linear(self, x, w: LinearWeight, out, bias=None, accumulate=False) -> None:
         """out (+)= x @ w.T + bias."""
-        if w.tiled is not None and x.shape[0] <= SKINNY_ROWS:
+        if w.tiled is not None:
             ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, bias=bias, accumulate=accumulate)
         else:
             ops.gemm(x, w.dense, out, bias=bias, accumulate=accumulate)
@@ -71,9 +70,19 @@ class Runtime:
                       cache.v_pool, cache.page_size, spec.window, spec.scale)
 
 
+def bucket(n: int, floor: int = 1) -> int:
+    """The power of two (at least `floor`) that n rounds up to."""
+    b = floor
+    while b < n:
+        b *= 2
+    return b
+
+
 def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
     """Wavefronts per (sequence, key/value head): enough to fill the chip
-    (about 2048 in all), each with at least 128 keys."""
-    want = -(-2048 // max(1, num_seqs * kv_heads))
-    most = max(1, max_ctx // 128)
+    (about 2048 in all), each with at least 128 keys.  Both inputs are rounded
+    up to powers of two first, so a step gives the same result whether it runs
+    kernel by kernel or as a graph captured for its bucket."""
+    want = -(-2048 // (bucket(num_seqs) * kv_heads))
+    most = max(1, bucket(max_ctx, 256) // 128)
     return max(1, min(want, most, 64))

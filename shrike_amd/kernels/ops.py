@@ -125,7 +125,8 @@ def retile_weight(w: torch.Tensor) -> torch.Tensor:
 
 
 def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False) -> None:
-    """out (+)= a @ w.T + bias for at most 64 rows of a; wt = retile_weight(w)."""
+    """out (+)= a @ w.T + bias with wt = retile_weight(w): up to 64 rows of a
+    stream the weights once; more rows run the LDS-staged MFMA kernel."""
     _rows(a, "gemm a")
     _rows(out, "gemm out")
     n = a.shape[0]

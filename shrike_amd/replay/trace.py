@@ -30,6 +30,7 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
+    ap.add_argument("--no-graphs", action="store_true", help="launch every step kernel by kernel")
     args = ap.parse_args(argv)
 
     out_dir = Path(args.out)
@@ -53,7 +54,7 @@ def main(argv=None) -> int:
     cache = CacheManager(model.cache_specs(), page, num_pages, max_slots=64,
                          enable_prefix_caching=False)
     cache.allocate(runtime.dtype, runtime.device)
-    runner = ModelRunner(model, cache, runtime)
+    runner = ModelRunner(model, cache, runtime, graphs=not args.no_graphs)
     _say(f"ready: {num_pages} pages of {page} tokens")
 
     live: dict[str, tuple] = {}  # id -> (SequenceCache, tokens so far)

@@ -369,11 +369,13 @@ def test_sample_frequencies_follow_the_distribution(ops):
 @pytest.mark.parametrize(
     "n, m, k",
     [(1, 48, 64), (8, 3584, 3584), (7, 503, 128), (16, 100, 172), (17, 130, 96), (33, 200, 333),
-     (48, 64, 64), (64, 1000, 520), (5, 37, 50)],
+     (48, 64, 64), (64, 1000, 520), (5, 37, 50), (65, 128, 64), (130, 200, 333), (300, 503, 128),
+     (1000, 172, 96), (257, 130, 172), (2048, 1024, 512)],
 )
 def test_gemm_tiled_weight(ops, n, m, k):
-    """The weight-streaming MFMA kernel over the tiled weight layout, at sizes
-    that are no multiple of the 16 x 32 tile and rows that are not 16-byte aligned."""
+    """The MFMA kernels over the tiled weight layout (weight-streaming up to 64
+    rows, LDS-staged above), at sizes that are no multiple of the tiles and
+    rows that are not 16-byte aligned."""
     torch.manual_seed(12)
     dtype = torch.bfloat16
     a, w, b = torch.randn(n, k), torch.randn(m, k) / math.sqrt(k), torch.randn(m)
