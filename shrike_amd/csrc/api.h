@@ -5,6 +5,7 @@
 // nothing was launched.  Shapes are checked on the host before any launch.
 #pragma once
 
+#include <stddef.h>
 #include <stdint.h>
 
 #ifdef __cplusplus
@@ -22,10 +23,11 @@ int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int 
 // when `rows` is given, else r):  x = resid[row] (+ delta[row]);  if
 // write_resid the sum is stored back into resid;  out[r] = x * rsqrt(mean(x^2)
 // + eps) * weight.  resid is float32, delta and out have `dtype`, weight is
-// float32.
+// float32.  delta_splits > 0: delta is float32 [delta_splits][resid rows][hidden],
+// partial sums of a product split along k, added in order.
 int shk_add_rmsnorm(float* resid, const void* delta, const float* weight, float eps, void* out,
                     int dtype, const int32_t* rows, int n, int hidden, int write_resid,
-                    void* stream);
+                    int delta_splits, int resid_rows, void* stream);
 
 // out[i, j] = silu(gu[i, j]) * gu[i, inter + j] for j < inter; gu is [n, 2*inter].
 int shk_silu_mul(const void* gu, void* out, int dtype, int n, int inter, void* stream);
@@ -42,11 +44,24 @@ int shk_gemm(const void* a, const void* w, const float* bias, void* out, int n, 
 // gemm_bf16.hip): ceil(m/16) * ceil(k/32) tiles of 1 KiB.
 int shk_retile_weight(const void* w, int m, int k, void* wt, void* stream);
 
+// wt = the tiled layouts of a gated feed-forward's gate and up matrices ([m, k]
+// each, given tiled) interleaved by blocks of 16 rows.
+int shk_interleave_gate_up(const void* gate_t, const void* up_t, int m, int k, void* wt,
+                           void* stream);
+
 // out[n, m] (+)= a[n, k] @ w^T + bias with w given in the tiled layout; a is
 // bfloat16 row-major with row stride lda; out is bfloat16 or float32.
+// gated: wt is an interleaved gate/up pair and out[n, m] = silu(a @ gate^T) *
+// (a @ up^T), without bias or accumulation.
+// ksplit > 1 (at most 64 rows, float32 output, no bias): the k range is shared
+// by ksplit workgroups per block of weight rows and out is [ksplit][n][m], the
+// partial sums, which the kernel that reads the product adds up in order
+// (shk_add_rmsnorm, shk_rope_kv_store).  shk_gemm_bf16_splits says how many
+// shares fill the chip for a shape (1: do not split).
 int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const float* bias, void* out, int n,
                                int m, int k, int lda, int ldo, int out_dtype, int accumulate,
-                               void* stream);
+                               int gated, int ksplit, void* stream);
+int shk_gemm_bf16_splits(int n, int m, int k);
 
 // Position encoding and cache write for the n tokens of a step.  qkv is
 // [n, (heads + 2*kv_heads) * head_dim]: queries, keys, values.  Queries and
@@ -56,11 +71,15 @@ int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const float* bias,
 // The key pool is [num_pages, kv_heads, page_size, head_dim]; the value pool is
 // stored transposed, [num_pages, kv_heads, head_dim, page_size].  rot_dim 0
 // rotates nothing; write_kv 0 leaves the pools alone.
+// splits > 0: the projections come as float32 partial sums `parts`
+// [splits][n][width] of a product split along k; they are added in order, `bias`
+// (float32 [width] or null) is added, and the rotated queries are written to
+// qkv's query columns (qkv is then output only).
 int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_heads, int head_dim,
                       int rot_dim, const float* inv_freq, const int32_t* positions,
                       const int32_t* token_seq, const int32_t* tables, int table_stride,
                       void* k_pool, void* v_pool, int page_size, int num_pages, int write_kv,
-                      void* stream);
+                      const float* parts, int splits, const float* bias, void* stream);
 
 // Causal attention of n query tokens over their sequences' paged caches.
 // Token t (position p, sequence s) reads keys j in (p - window, p] (all j <= p

@@ -43,10 +43,60 @@ struct TileArgs {
   float scale;
 };
 
+// The operands of one chunk of 32 keys: K rows for two score tiles and the
+// transposed V columns for P.V.
+template <int D>
+struct Chunk {
+  AFrag k[2][D / 32];
+  AFrag v[D / 16];
+};
+
+// Issues every load of the chunk at key `kb`; tiles and key groups that no row
+// reads (beyond pos_max, before lo_min) are not touched and read as zero.
+template <int D>
+__device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, int kb, int pos_max,
+                                           int lo_min) {
+  const int lane = threadIdx.x % kWave;
+  const int j = lane % 16, kg = lane / 16;
+  const int ps = ta.page_size;
+  const size_t head_elems = static_cast<size_t>(ps) * D;  // one kv head of one page
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    const int key0 = kb + tt * 16;
+    const bool live = key0 <= pos_max && key0 + 15 >= lo_min;
+    const bf16* krow = nullptr;
+    if (live) {
+      const int page = ta.table[key0 / ps];
+      krow = ta.k_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
+             static_cast<size_t>(key0 % ps + j) * D + kg * 8;
+    }
+#pragma unroll
+    for (int ds = 0; ds < D / 32; ++ds) {
+      c.k[tt][ds].u = make_uint4(0, 0, 0, 0);
+      if (live) c.k[tt][ds].u = *reinterpret_cast<const uint4*>(krow + ds * 32);
+    }
+  }
+  // this lane supplies keys kb + 8*kg .. +8 of element db*16 + j
+  const int g0 = kb + kg * 8;
+  const bool live = g0 <= pos_max && g0 + 7 >= lo_min;
+  const bf16* vcol = nullptr;
+  if (live) {
+    const int page = ta.table[g0 / ps];
+    vcol = ta.v_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
+           static_cast<size_t>(j) * ps + g0 % ps;
+  }
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) {
+    c.v[db].u = make_uint4(0, 0, 0, 0);
+    if (live) c.v[db].u = *reinterpret_cast<const uint4*>(vcol + static_cast<size_t>(db) * 16 * ps);
+  }
+}
+
 // Walks keys [key_begin, key_end) (key_begin a multiple of 32) for 16 rows.
 // qf: the rows' queries as A operands.  row_pos / row_lo: for this lane's four
 // accumulator rows (4*(lane/16) + r), the last and first key each may read.
-// pos_max / lo_min: the same bounds over all 16 rows.
+// pos_max / lo_min: the same bounds over all 16 rows.  The next chunk's loads
+// are in flight while the current chunk is computed.
 template <int D>
 __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf)[D / 32],
                                             const int (&row_pos)[4], const int (&row_lo)[4],
@@ -55,26 +105,20 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
                                             uint16_t* p_lds) {
   const int lane = threadIdx.x % kWave;
   const int j = lane % 16, kg = lane / 16;
-  const int ps = ta.page_size;
-  const size_t head_elems = static_cast<size_t>(ps) * D;  // one kv head of one page
 
+  Chunk<D> cur, nxt;
+  if (key_begin < key_end) load_chunk<D>(cur, ta, key_begin, pos_max, lo_min);
   for (int kb = key_begin; kb < key_end; kb += 32) {
+    if (kb + 32 < key_end) load_chunk<D>(nxt, ta, kb + 32, pos_max, lo_min);
+
     // ---- S = Q K^T for two tiles of 16 keys
     f32x4 s[2];
 #pragma unroll
     for (int tt = 0; tt < 2; ++tt) {
       s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      const int key0 = kb + tt * 16;
-      if (key0 > pos_max || key0 + 15 < lo_min) continue;  // no row reads this tile
-      const int page = ta.table[key0 / ps];
-      const bf16* krow = ta.k_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
-                         static_cast<size_t>(key0 % ps + j) * D + kg * 8;
-      AFrag kf[D / 32];
-#pragma unroll
-      for (int ds = 0; ds < D / 32; ++ds) kf[ds].u = *reinterpret_cast<const uint4*>(krow + ds * 32);
 #pragma unroll
       for (int ds = 0; ds < D / 32; ++ds)
-        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ds].v, kf[ds].v, s[tt], 0, 0, 0);
+        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ds].v, cur.k[tt][ds].v, s[tt], 0, 0, 0);
     }
 
     // ---- mask, running maximum and sum (lane holds key kb + tt*16 + j for rows 4*kg + r)
@@ -116,18 +160,11 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
     AFrag pf;
     pf.u = *reinterpret_cast<const uint4*>(p_lds + j * kPStride + kg * 8);
 
-    // ---- O += P V: this lane supplies keys kb + 8*kg .. +8 of element db*16 + j
+    // ---- O += P V.  Keys outside [lo_min, pos_max] carry weight 0 but their
+    // slots may hold anything: zero them so that 0 * x stays 0.
     const int g0 = kb + kg * 8;
-    const bool live = g0 <= pos_max && g0 + 7 >= lo_min;
-    const bf16* vcol = nullptr;
-    if (live) {
-      const int page = ta.table[g0 / ps];
-      vcol = ta.v_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
-             static_cast<size_t>(j) * ps + g0 % ps;
-    }
-    // keys outside [lo_min, pos_max] carry weight 0 but may hold anything: zero them
     uint4 keep_bits = make_uint4(~0u, ~0u, ~0u, ~0u);
-    if (live && (g0 < lo_min || g0 + 7 > pos_max)) {
+    if (g0 < lo_min || g0 + 7 > pos_max) {
       uint32_t w[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -139,17 +176,14 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
     }
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) {
-      AFrag vf;
-      vf.u = make_uint4(0, 0, 0, 0);
-      if (live) {
-        vf.u = *reinterpret_cast<const uint4*>(vcol + static_cast<size_t>(db) * 16 * ps);
-        vf.u.x &= keep_bits.x;
-        vf.u.y &= keep_bits.y;
-        vf.u.z &= keep_bits.z;
-        vf.u.w &= keep_bits.w;
-      }
+      AFrag vf = cur.v[db];
+      vf.u.x &= keep_bits.x;
+      vf.u.y &= keep_bits.y;
+      vf.u.z &= keep_bits.z;
+      vf.u.w &= keep_bits.w;
       o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, o[db], 0, 0, 0);
     }
+    cur = nxt;
   }
 }
 
@@ -220,23 +254,32 @@ __global__ void __launch_bounds__(kWave)
 }
 
 // out[seq][head][:] = sum_z exp(m_z - M) O_z / sum_z exp(m_z - M) l_z, splits in order.
+constexpr int kMaxSplits = 64;
+
 __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
                                        int head_dim, int nsplit) {
+  __shared__ float ms[kMaxSplits], ls[kMaxSplits];
   const size_t row = blockIdx.x;  // seq * heads + head
-  const float* src = partial + row * nsplit * (head_dim + 2);
+  const int stride = head_dim + 2;
+  const float* src = partial + row * nsplit * stride;
+  if (threadIdx.x < nsplit) {
+    ms[threadIdx.x] = src[threadIdx.x * stride + head_dim];
+    ls[threadIdx.x] = src[threadIdx.x * stride + head_dim + 1];
+  }
+  __syncthreads();
   float mx = -INFINITY;
-  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, src[z * (head_dim + 2) + head_dim]);
+  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, ms[z]);
+  float den = 0.f;
+  for (int z = 0; z < nsplit; ++z) den += (ms[z] == -INFINITY ? 0.f : __expf(ms[z] - mx)) * ls[z];
+  const float inv = 1.f / den;
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float num = 0.f, den = 0.f;
+    float num = 0.f;
+#pragma unroll 8
     for (int z = 0; z < nsplit; ++z) {
-      const float* pz = src + z * (head_dim + 2);
-      const float mz = pz[head_dim];
-      if (mz == -INFINITY) continue;
-      const float f = __expf(mz - mx);
-      num += f * pz[d];
-      den += f * pz[head_dim + 1];
+      const float f = ms[z] == -INFINITY ? 0.f : __expf(ms[z] - mx);
+      num += f * src[z * stride + d];
     }
-    out[row * head_dim + d] = from_float<bf16>(num / den);
+    out[row * head_dim + d] = from_float<bf16>(num * inv);
   }
 }
 
@@ -372,8 +415,9 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
                                          int nsplit, void* stream) {
   if (check_mfma_shapes("attention_decode", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
   SHK_REQUIRE(heads / kv_heads <= 16, "attention_decode: at most 16 query heads per key/value head");
-  SHK_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && nsplit >= 1 && nsplit <= 65535,
-              "attention_decode: bad sizes num_seqs=%d nsplit=%d", num_seqs, nsplit);
+  SHK_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && nsplit >= 1 && nsplit <= kMaxSplits,
+              "attention_decode: bad sizes num_seqs=%d nsplit=%d (at most %d splits)", num_seqs,
+              nsplit, kMaxSplits);
   if (num_seqs == 0) return 0;
   SHK_REQUIRE(q && out && positions && tables && k_pool && v_pool && partial && table_stride > 0,
               "attention_decode: null pointer");

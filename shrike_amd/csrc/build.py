@@ -35,7 +35,7 @@ HIPCC_FLAGS = [
     "-Xclang",
     "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
-]
+] + os.environ.get("SHRIKE_HIPCC_EXTRA", "").split()
 
 
 def sources() -> list[Path]:

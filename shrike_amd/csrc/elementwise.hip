@@ -29,10 +29,84 @@ __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restr
 }
 
 // ------------------------------------------------------------ add + RMSNorm
-// One workgroup per row.  The row is read once into registers when it fits
-// (hidden <= 256 * kMaxPerThread), otherwise it is re-read from resid.
+// One workgroup per row.  add_rmsnorm_vec_kernel holds the row in registers
+// (hidden a multiple of 4, at most 256 * 4 * kNormVecs elements): all loads
+// are issued before the first use, so a row costs one memory round trip.
+// add_rmsnorm_kernel takes every other size.
 
 constexpr int kNormThreads = 256;
+constexpr int kNormVecs = 8;  // float4 per thread: rows of up to 8192 elements
+
+__device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 load4(const bf16* p) {
+  const uint2 u = *reinterpret_cast<const uint2*>(p);
+  return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                     __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+}
+__device__ __forceinline__ void store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16* p, float4 v) {
+  uint2 u;
+  u.x = bf16_bits(v.x) | (static_cast<uint32_t>(bf16_bits(v.y)) << 16);
+  u.y = bf16_bits(v.z) | (static_cast<uint32_t>(bf16_bits(v.w)) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+// TD is the type of delta: T, or float for the partial sums of a split product
+// ([splits][resid_rows][hidden], added in order).
+template <typename T, typename TD>
+__global__ void __launch_bounds__(kNormThreads)
+    add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
+                           const float* __restrict__ weight, float eps, T* __restrict__ out,
+                           const int32_t* __restrict__ rows, int hidden, int write_resid,
+                           int splits, size_t split_stride) {
+  __shared__ float scratch[16];
+  const int r = blockIdx.x;
+  const size_t row = rows ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
+  float* x = resid + row * hidden;
+  const TD* d = delta ? delta + row * hidden : nullptr;
+  T* y = out + static_cast<size_t>(r) * hidden;
+  const int nvec = hidden / 4;
+
+  float4 v[kNormVecs], dv[kNormVecs], w[kNormVecs];
+#pragma unroll
+  for (int i = 0; i < kNormVecs; ++i) {
+    const int c = threadIdx.x + i * kNormThreads;
+    v[i] = dv[i] = w[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (c < nvec) {
+      v[i] = load4(x + c * 4);
+      if (d) dv[i] = load4(d + c * 4);
+      w[i] = load4(weight + c * 4);
+    }
+  }
+  for (int z = 1; z < splits; ++z) {
+    float4 more[kNormVecs];
+#pragma unroll
+    for (int i = 0; i < kNormVecs; ++i) {
+      const int c = threadIdx.x + i * kNormThreads;
+      more[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (c < nvec) more[i] = load4(d + z * split_stride + c * 4);
+    }
+#pragma unroll
+    for (int i = 0; i < kNormVecs; ++i)
+      dv[i].x += more[i].x, dv[i].y += more[i].y, dv[i].z += more[i].z, dv[i].w += more[i].w;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < kNormVecs; ++i) {
+    v[i].x += dv[i].x, v[i].y += dv[i].y, v[i].z += dv[i].z, v[i].w += dv[i].w;
+    ss += v[i].x * v[i].x + v[i].y * v[i].y + v[i].z * v[i].z + v[i].w * v[i].w;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
+#pragma unroll
+  for (int i = 0; i < kNormVecs; ++i) {
+    const int c = threadIdx.x + i * kNormThreads;
+    if (c >= nvec) continue;
+    if (d && write_resid) store4(x + c * 4, v[i]);
+    store4(y + c * 4, make_float4((v[i].x * inv) * w[i].x, (v[i].y * inv) * w[i].y,
+                                  (v[i].z * inv) * w[i].z, (v[i].w * inv) * w[i].w));
+  }
+}
 
 template <typename T>
 __global__ void __launch_bounds__(kNormThreads)
@@ -103,21 +177,42 @@ extern "C" int shk_embed(const void* table, int dtype, const int32_t* ids, float
 
 extern "C" int shk_add_rmsnorm(float* resid, const void* delta, const float* weight, float eps,
                                void* out, int dtype, const int32_t* rows, int n, int hidden,
-                               int write_resid, void* stream) {
+                               int write_resid, int delta_splits, int resid_rows, void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "add_rmsnorm: unknown dtype %d", dtype);
   SHK_REQUIRE(n >= 0 && hidden > 0, "add_rmsnorm: bad sizes n=%d hidden=%d", n, hidden);
   SHK_REQUIRE(eps > 0.f, "add_rmsnorm: eps must be > 0");
   if (n == 0) return 0;
   SHK_REQUIRE(resid && weight && out, "add_rmsnorm: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (dtype == kF32)
-    add_rmsnorm_kernel<float><<<n, kNormThreads, 0, s>>>(
-        resid, static_cast<const float*>(delta), weight, eps, static_cast<float*>(out), rows,
-        hidden, write_resid);
-  else
-    add_rmsnorm_kernel<bf16><<<n, kNormThreads, 0, s>>>(
-        resid, static_cast<const bf16*>(delta), weight, eps, static_cast<bf16*>(out), rows, hidden,
-        write_resid);
+  const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = hidden % 4 == 0 && hidden <= kNormThreads * 4 * kNormVecs && aligned(resid) &&
+                   aligned(weight) && aligned(out) && (!delta || aligned(delta));
+  if (delta_splits > 0) {
+    SHK_REQUIRE(delta && vec && dtype == kBF16 && resid_rows > 0,
+                "add_rmsnorm: partial sums need bfloat16 output, hidden %% 4 == 0 and at most %d",
+                kNormThreads * 4 * kNormVecs);
+    add_rmsnorm_vec_kernel<bf16, float><<<n, kNormThreads, 0, s>>>(
+        resid, static_cast<const float*>(delta), weight, eps, static_cast<bf16*>(out), rows, hidden,
+        write_resid, delta_splits, static_cast<size_t>(resid_rows) * hidden);
+  } else if (dtype == kF32) {
+    if (vec)
+      add_rmsnorm_vec_kernel<float, float><<<n, kNormThreads, 0, s>>>(
+          resid, static_cast<const float*>(delta), weight, eps, static_cast<float*>(out), rows,
+          hidden, write_resid, 1, 0);
+    else
+      add_rmsnorm_kernel<float><<<n, kNormThreads, 0, s>>>(
+          resid, static_cast<const float*>(delta), weight, eps, static_cast<float*>(out), rows,
+          hidden, write_resid);
+  } else {
+    if (vec)
+      add_rmsnorm_vec_kernel<bf16, bf16><<<n, kNormThreads, 0, s>>>(
+          resid, static_cast<const bf16*>(delta), weight, eps, static_cast<bf16*>(out), rows,
+          hidden, write_resid, 1, 0);
+    else
+      add_rmsnorm_kernel<bf16><<<n, kNormThreads, 0, s>>>(
+          resid, static_cast<const bf16*>(delta), weight, eps, static_cast<bf16*>(out), rows,
+          hidden, write_resid);
+  }
   SHK_LAUNCH_CHECK("add_rmsnorm");
   return 0;
 }

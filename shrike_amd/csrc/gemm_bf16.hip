@@ -8,10 +8,10 @@
 // so the operand of one MFMA is one fully coalesced 1 KiB load and a block of
 // 16 rows streams as one contiguous region.
 //
-// gemm_skinny_kernel: for few tokens (decode).  One workgroup of 4 wavefronts
-// per block of 16 weight rows; the wavefronts take the k-tiles round-robin and
-// their partial sums are added in a fixed order through LDS.  The weights are
-// read exactly once from HBM; accumulation is float32.
+// gemm_skinny_kernel: for few tokens (decode).  One workgroup of 4, 8 or 16
+// wavefronts per block of 16 weight rows; the wavefronts take the k-tiles
+// round-robin and their partial sums are added in a fixed order through LDS.
+// The weights are read exactly once from HBM; accumulation is float32.
 #include "api.h"
 #include "common.h"
 
@@ -45,79 +45,132 @@ __device__ __forceinline__ Frag load_act(const bf16* __restrict__ a, int lda, in
   return f;
 }
 
-constexpr int kSkinnyWaves = 4;
-constexpr int kSkinnyUnroll = 8;
+constexpr int kSkinnyBatch = 4;  // k-tiles a wavefront has in flight per buffer
 
-template <int NB>
-__global__ void __launch_bounds__(kSkinnyWaves* kWave)
+// One batch of operands: kSkinnyBatch weight tiles and the matching activations.
+// (RB = 2 for the gated variant: the tiles of a gate block and of its up block.)
+template <int NB, int RB>
+struct SkinnyBatch {
+  Frag w[kSkinnyBatch][RB];
+  Frag x[kSkinnyBatch][NB];
+};
+
+__device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); }
+
+template <int NB, int RB>
+__device__ __forceinline__ void skinny_load(SkinnyBatch<NB, RB>& b, const uint4* __restrict__ wrow,
+                                            const bf16* __restrict__ a, int lda, int n, int k,
+                                            int ktiles, int t, int step, int j, int kg, bool vec) {
+#pragma unroll
+  for (int u = 0; u < kSkinnyBatch; ++u) {
+    const int tt = t + u * step;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      b.w[u][rb].u = make_uint4(0, 0, 0, 0);
+      // weights are read once: a non-temporal load keeps them from displacing
+      // the activations in the caches
+      if (tt < ktiles) {
+        const uint4* p = wrow + (static_cast<size_t>(rb) * ktiles + tt) * kWave;
+        b.w[u][rb].u.x = __builtin_nontemporal_load(&p->x);
+        b.w[u][rb].u.y = __builtin_nontemporal_load(&p->y);
+        b.w[u][rb].u.z = __builtin_nontemporal_load(&p->z);
+        b.w[u][rb].u.w = __builtin_nontemporal_load(&p->w);
+      }
+    }
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+      b.x[u][nb] = load_act(a, lda, n, k, nb * 16 + j, tt * 32 + kg * 8, vec);
+  }
+}
+
+// WAVES wavefronts per workgroup share one block of 16 weight rows and take
+// its k-tiles round-robin (wavefront w: tiles w, w + WAVES, ...), so the
+// workgroup reads contiguous stretches of the block.  Each wavefront keeps two
+// batches of tiles in registers: the next batch is in flight while the current
+// one is multiplied.  The host picks WAVES so that about 4096 wavefronts or
+// more are in flight whatever the number of rows.
+//
+// GATED: the weight holds a gated feed-forward's two matrices interleaved by
+// blocks of 16 rows (block 2b: rows 16b.. of the gate matrix, block 2b+1: the
+// same rows of the up matrix).  A workgroup multiplies both blocks and writes
+// silu(gate) * up: out[token][16b + row], `m` being the width of that output.
+template <int NB, int WAVES, bool GATED>
+__global__ void __launch_bounds__(WAVES* kWave)
     gemm_skinny_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                        const uint4* __restrict__ wt, int ktiles, int m,
                        const float* __restrict__ bias, void* __restrict__ out, int ldo,
-                       int out_f32, int accumulate, int vec) {
-  __shared__ float red[kSkinnyWaves][NB][kWave][4];
+                       int out_f32, int accumulate, int vec, int ksplit) {
+  constexpr int RB = GATED ? 2 : 1;
+  __shared__ float red[WAVES][RB][NB][kWave][4];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int mb = blockIdx.x;
+  const int mb = blockIdx.x;  // block of 16 output rows
+  const int z = blockIdx.y;   // which share of k (ksplit workgroups per block)
   const int j = lane % 16, kg = lane / 16;
-  const uint4* wrow = wt + static_cast<size_t>(mb) * ktiles * kWave + lane;
+  const uint4* wrow = wt + static_cast<size_t>(mb) * RB * ktiles * kWave + lane;
 
-  f32x4 acc[NB];
+  f32x4 acc[RB][NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[rb][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // k-tiles wave, wave + 4, ...; kSkinnyUnroll of them in flight at a time
-  int t = wave;
-  for (; t + (kSkinnyUnroll - 1) * kSkinnyWaves < ktiles; t += kSkinnyUnroll * kSkinnyWaves) {
-    Frag w[kSkinnyUnroll];
+  // k-tile t belongs to wavefront (t % (WAVES * ksplit)) of the block's ksplit workgroups
+  SkinnyBatch<NB, RB> cur, next;
+  const int lanes_k = WAVES * ksplit;  // wavefronts that share the block's k-tiles
+  const int kStride = kSkinnyBatch * lanes_k;
+  const int t0 = z * WAVES + wave;
+  skinny_load<NB, RB>(cur, wrow, a, lda, n, k, ktiles, t0, lanes_k, j, kg, vec);
+  for (int t = t0; t < ktiles; t += kStride) {
+    if (t + kStride < ktiles)
+      skinny_load<NB, RB>(next, wrow, a, lda, n, k, ktiles, t + kStride, lanes_k, j, kg, vec);
 #pragma unroll
-    for (int u = 0; u < kSkinnyUnroll; ++u)
-      w[u].u = wrow[static_cast<size_t>(t + u * kSkinnyWaves) * kWave];
+    for (int u = 0; u < kSkinnyBatch; ++u)
 #pragma unroll
-    for (int u = 0; u < kSkinnyUnroll; ++u) {
-      const int kk = (t + u * kSkinnyWaves) * 32 + kg * 8;
+      for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        const Frag x = load_act(a, lda, n, k, b * 16 + j, kk, vec);
-        acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u].v, x.v, acc[b], 0, 0, 0);
-      }
-    }
-  }
-  for (; t < ktiles; t += kSkinnyWaves) {
-    Frag w;
-    w.u = wrow[static_cast<size_t>(t) * kWave];
-    const int kk = t * 32 + kg * 8;
-#pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      const Frag x = load_act(a, lda, n, k, b * 16 + j, kk, vec);
-      acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w.v, x.v, acc[b], 0, 0, 0);
-    }
+        for (int b = 0; b < NB; ++b)
+          acc[rb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.w[u][rb].v, cur.x[u][b].v,
+                                                               acc[rb][b], 0, 0, 0);
+    cur = next;
   }
 
 #pragma unroll
-  for (int b = 0; b < NB; ++b)
+  for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) red[wave][b][lane][r] = acc[b][r];
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) red[wave][rb][b][lane][r] = acc[rb][b][r];
   __syncthreads();
 
-  // Lane (j, kg) of accumulator b holds rows kg*4 + r of the block for token b*16 + j.
-  // Wavefront w finishes the token blocks b = w, w + 4, ...
-  for (int b = wave; b < NB; b += kSkinnyWaves) {
-    const int token = b * 16 + j;
-    if (token >= n) continue;
+  // Element e of the block's 16 x (16 * NB) outputs: accumulator b = e / 256,
+  // lane (e % 256) / 4, register r = e % 4.  Lane (j, kg) holds rows kg*4 + r
+  // for token b*16 + j.  The wavefronts' partial sums are added in wavefront order.
+  for (int e = threadIdx.x; e < NB * 256; e += WAVES * kWave) {
+    const int b = e / 256, ln = (e % 256) / 4, r = e % 4;
+    const int token = b * 16 + ln % 16, row = mb * 16 + (ln / 16) * 4 + r;
+    if (token >= n || row >= m) continue;
+    float v = red[0][0][b][ln][r], up = 0.f;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int row = mb * 16 + kg * 4 + r;
-      if (row >= m) continue;
-      float v = red[0][b][lane][r];
+    for (int w = 1; w < WAVES; ++w) v += red[w][0][b][ln][r];
+    if (ksplit > 1) {
+      // this workgroup's share of k: a float32 partial sum, [ksplit][n][m], that the
+      // kernel which reads the product adds up in order
+      static_cast<float*>(out)[(static_cast<size_t>(z) * n + token) * ldo + row] = v;
+      continue;
+    }
+    if (GATED) {
+      up = red[0][RB - 1][b][ln][r];
 #pragma unroll
-      for (int w = 1; w < kSkinnyWaves; ++w) v += red[w][b][lane][r];
-      if (bias) v += bias[row];
-      const size_t idx = static_cast<size_t>(token) * ldo + row;
-      if (out_f32) {
-        float* o = static_cast<float*>(out);
-        o[idx] = accumulate ? o[idx] + v : v;
-      } else {
-        static_cast<bf16*>(out)[idx] = from_float<bf16>(v);
-      }
+      for (int w = 1; w < WAVES; ++w) up += red[w][RB - 1][b][ln][r];
+    }
+    if (GATED) v = silu(v) * up;
+    if (bias) v += bias[row];
+    const size_t idx = static_cast<size_t>(token) * ldo + row;
+    if (out_f32) {
+      float* o = static_cast<float*>(out);
+      o[idx] = accumulate ? o[idx] + v : v;
+    } else {
+      static_cast<bf16*>(out)[idx] = from_float<bf16>(v);
     }
   }
 }
@@ -136,6 +189,7 @@ constexpr int kBigN = 128;   // tokens per workgroup
 constexpr int kBigK = 64;    // k per stage (two MFMA steps)
 constexpr int kBigFrags = (kBigM / 16) * (kBigK / 32);  // fragments per operand per stage: 16
 
+template <bool GATED>
 __global__ void __launch_bounds__(256)
     gemm_big_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                     const uint4* __restrict__ wt, int ktiles, int m,
@@ -147,7 +201,8 @@ __global__ void __launch_bounds__(256)
   const int wm = wave / 2, wn = wave % 2;  // quadrant of the wavefront
   const int mb0 = blockIdx.x * (kBigM / 16);   // first block of 16 weight rows
   const int tok0 = blockIdx.y * kBigN;
-  const int mblocks = (m + 15) / 16;
+  // blocks of 16 weight rows; a gated weight has two per 16 output rows
+  const int mblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
   const int nstages = (ktiles + 1) / 2;
 
   f32x4 acc[4][4];
@@ -211,13 +266,14 @@ __global__ void __launch_bounds__(256)
     const int token = tok0 + (wn * 4 + jn) * 16 + j;
     if (token >= n) continue;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int row0 = (mb0 + wm * 4 + i) * 16 + kg * 4;
+    for (int i = 0; i < 4; i += (GATED ? 2 : 1)) {
+      // gated: weight blocks come in (gate, up) pairs that make one block of output rows
+      const int row0 = (GATED ? (mb0 + wm * 4 + i) / 2 : mb0 + wm * 4 + i) * 16 + kg * 4;
       if (row0 >= m) continue;
       float v[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        v[r] = acc[i][jn][r];
+        v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r] : acc[i][jn][r];
         if (bias && row0 + r < m) v[r] += bias[row0 + r];
       }
       const size_t idx = static_cast<size_t>(token) * ldo + row0;
@@ -273,9 +329,53 @@ extern "C" int shk_retile_weight(const void* w, int m, int k, void* wt, void* st
   return 0;
 }
 
+// Interleaves the tiled layouts of a gate and an up matrix ([m, k] each) by
+// blocks of 16 rows: wt[2b] = gate block b, wt[2b + 1] = up block b.
+__global__ void interleave_blocks_kernel(const uint4* __restrict__ gate, const uint4* __restrict__ up,
+                                         uint4* __restrict__ wt, size_t block_vecs) {
+  const size_t b = blockIdx.y;
+  for (size_t i = blockIdx.x * blockDim.x + threadIdx.x; i < block_vecs;
+       i += static_cast<size_t>(gridDim.x) * blockDim.x) {
+    wt[(2 * b) * block_vecs + i] = gate[b * block_vecs + i];
+    wt[(2 * b + 1) * block_vecs + i] = up[b * block_vecs + i];
+  }
+}
+
+extern "C" int shk_interleave_gate_up(const void* gate_t, const void* up_t, int m, int k, void* wt,
+                                      void* stream) {
+  SHK_REQUIRE(m > 0 && k > 0 && gate_t && up_t && wt, "interleave_gate_up: bad arguments");
+  const int mb = (m + 15) / 16, kt = (k + 31) / 32;
+  SHK_REQUIRE(mb <= 65535, "interleave_gate_up: too many rows (%d)", m);
+  const size_t block_vecs = static_cast<size_t>(kt) * kWave;
+  interleave_blocks_kernel<<<dim3(8, mb), 256, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const uint4*>(gate_t), static_cast<const uint4*>(up_t), static_cast<uint4*>(wt),
+      block_vecs);
+  SHK_LAUNCH_CHECK("interleave_gate_up");
+  return 0;
+}
+
+// Workgroups per block of 16 weight rows that a product with at most 64 rows
+// should be split into along k so that the chip is full (about 8192 wavefronts
+// with 4 k-tiles or more each): 1 for matrices with many row blocks.
+extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
+  const int mblocks = (m + 15) / 16, ktiles = (k + 31) / 32;
+  if (n > 64 || mblocks >= 512) return 1;
+  int split = 8192 / (mblocks * 4);
+  const int most = ktiles / 16;
+  if (split > most) split = most;
+  if (split > 16) split = 16;
+  return split > 1 ? split : 1;
+}
+
 extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const float* bias,
                                           void* out, int n, int m, int k, int lda, int ldo,
-                                          int out_dtype, int accumulate, void* stream) {
+                                          int out_dtype, int accumulate, int gated, int ksplit,
+                                          void* stream) {
+  SHK_REQUIRE(!gated || (!accumulate && !bias), "gemm_bf16: a gated product takes no bias and does not accumulate");
+  SHK_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_bf16: ksplit %d is outside 1..64", ksplit);
+  SHK_REQUIRE(ksplit == 1 || (n <= 64 && !gated && !accumulate && !bias && out_dtype == kF32 && ldo == m),
+              "gemm_bf16: a product split along k has at most 64 rows and writes plain float32 "
+              "partial sums [ksplit][n][m]");
   SHK_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "gemm_bf16: unknown out_dtype %d",
               out_dtype);
   SHK_REQUIRE(n >= 0 && m > 0 && k > 0, "gemm_bf16: bad sizes n=%d m=%d k=%d", n, m, k);
@@ -293,14 +393,39 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
     dim3 grid((m + kBigM - 1) / kBigM, (n + kBigN - 1) / kBigN);
     SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);
-    gemm_big_kernel<<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate,
-                                         vec);
+    if (gated) {
+      grid.x = (2 * mb * 16 + kBigM - 1) / kBigM;
+      gemm_big_kernel<true><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,
+                                                 accumulate, vec);
+    } else {
+      gemm_big_kernel<false><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,
+                                                  accumulate, vec);
+    }
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }
-#define SHK_SKINNY(NB)                                                                        \
-  gemm_skinny_kernel<NB><<<mb, kSkinnyWaves * kWave, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, \
-                                                             out, ldo, of, accumulate, vec)
+  // wavefronts per workgroup: matrices with few row blocks get more of them
+  const int waves = (mb >= 512 || ksplit > 1) ? ((mb >= 512) ? 8 : 4) : 16;
+  const int max_waves = (n > 32 || (gated && n > 16)) ? 8 : 16;  // register budget of the wide variants
+  dim3 sgrid(mb, ksplit);
+#define SHK_SKINNY_W(NB, W)                                                                     \
+  do {                                                                                          \
+    if (gated)                                                                                  \
+      gemm_skinny_kernel<NB, W, true><<<sgrid, W * kWave, 0, s>>>(                              \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);               \
+    else                                                                                        \
+      gemm_skinny_kernel<NB, W, false><<<sgrid, W * kWave, 0, s>>>(                             \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);               \
+  } while (0)
+#define SHK_SKINNY(NB)                       \
+  do {                                       \
+    if (waves == 4)                          \
+      SHK_SKINNY_W(NB, 4);                   \
+    else if (waves == 8 || max_waves == 8)   \
+      SHK_SKINNY_W(NB, 8);                   \
+    else                                     \
+      SHK_SKINNY_W(NB, 16);                  \
+  } while (0)
   if (n <= 16)
     SHK_SKINNY(1);
   else if (n <= 32)
@@ -310,6 +435,7 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   else
     SHK_SKINNY(4);
 #undef SHK_SKINNY
+#undef SHK_SKINNY_W
   SHK_LAUNCH_CHECK("gemm_bf16");
   return 0;
 }

@@ -1,78 +1,99 @@
 // Rotary position encoding of queries and keys fused with the write of keys
-// and values into their cache pages.  One workgroup per token.  Angles, sine
-// and cosine are float32 (sincosf with full range reduction: positions reach
-// thousands of radians at the highest frequency).
+// and values into their cache pages.  One thread per element pair (queries and
+// keys) or element (values); a workgroup first tabulates the cosines and sines
+// of its token in LDS.  Angles, sine and cosine are float32 (sincosf with full
+// range reduction: positions reach thousands of radians at the highest
+// frequency).  The projections may arrive as the float32 partial sums of a
+// product that was split along k; they are added here, in order, with the bias.
 #include "api.h"
 #include "common.h"
 
 namespace shk {
 
 constexpr int kMaxHalf = 256;  // rot_dim / 2 <= 256
+constexpr int kRopeThreads = 256;
 
 template <typename T>
-__global__ void __launch_bounds__(256)
-    rope_kv_store_kernel(T* __restrict__ qkv, int heads, int kv_heads, int head_dim, int rot_dim,
-                         const float* __restrict__ inv_freq, const int32_t* __restrict__ positions,
+__global__ void __launch_bounds__(kRopeThreads)
+    rope_kv_store_kernel(T* __restrict__ qkv, int n, int heads, int kv_heads, int head_dim,
+                         int rot_dim, const float* __restrict__ inv_freq,
+                         const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ token_seq, const int32_t* __restrict__ tables,
                          int table_stride, T* __restrict__ k_pool, T* __restrict__ v_pool,
-                         int page_size, int num_pages, int write_kv) {
+                         int page_size, int num_pages, int write_kv,
+                         const float* __restrict__ parts, int splits,
+                         const float* __restrict__ bias) {
   __shared__ float cs[kMaxHalf];
   __shared__ float sn[kMaxHalf];
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot_dim / 2;
-  for (int i = threadIdx.x; i < half; i += blockDim.x) {
-    const float angle = static_cast<float>(pos) * inv_freq[i];
+  const int width = (heads + 2 * kv_heads) * head_dim;
+  for (int i = threadIdx.x; i < half; i += kRopeThreads) {
     float s, c;
-    sincosf(angle, &s, &c);
+    sincosf(static_cast<float>(pos) * inv_freq[i], &s, &c);
     cs[i] = c;
     sn[i] = s;
   }
   __syncthreads();
 
-  T* row = qkv + static_cast<size_t>(t) * (heads + 2 * kv_heads) * head_dim;
-  size_t slot_row = 0;  // index of this token's [head_dim] row for kv head 0
-  int page = 0;
+  T* row = qkv + static_cast<size_t>(t) * width;
+  // column `col` of this token's projections
+  auto in = [&](int col) -> float {
+    if (splits == 0) return to_float(row[col]);
+    const size_t split_stride = static_cast<size_t>(n) * width;
+    const float* p = parts + static_cast<size_t>(t) * width + col;
+    float v = p[0];
+    for (int z = 1; z < splits; ++z) v += p[z * split_stride];
+    return bias ? v + bias[col] : v;
+  };
+
+  int page = -1;
   if (write_kv) {
     page = tables[static_cast<size_t>(token_seq[t]) * table_stride + pos / page_size];
     // The host builds tables that cover every position of the step; a page id
     // outside the pool would be a host bug, and is never dereferenced.
-    if (page < 0 || page >= num_pages) write_kv = 0;
-    slot_row = (static_cast<size_t>(page) * kv_heads) * page_size + pos % page_size;
+    if (page < 0 || page >= num_pages) page = -1;
   }
-  const size_t head_rows = page_size;  // rows between consecutive kv heads of one page
+  const int slot = pos % page_size;
+  // keys [page][kv head][slot][head_dim]; values transposed [page][kv head][head_dim][slot]
+  const size_t page_base = static_cast<size_t>(page < 0 ? 0 : page) * kv_heads * page_size * head_dim;
 
-  // queries: rotate in place
-  for (int idx = threadIdx.x; idx < heads * half; idx += blockDim.x) {
-    const int h = idx / half, i = idx % half;
-    T* x = row + h * head_dim;
-    const float x1 = to_float(x[i]), x2 = to_float(x[i + half]);
-    x[i] = from_float<T>(x1 * cs[i] - x2 * sn[i]);
-    x[i + half] = from_float<T>(x2 * cs[i] + x1 * sn[i]);
-  }
-  if (!write_kv) return;
-
-  // keys: rotate into the page
-  const T* krow = row + heads * head_dim;
-  for (int idx = threadIdx.x; idx < kv_heads * half; idx += blockDim.x) {
-    const int h = idx / half, i = idx % half;
-    const T* x = krow + h * head_dim;
-    T* dst = k_pool + (slot_row + h * head_rows) * head_dim;
-    const float x1 = to_float(x[i]), x2 = to_float(x[i + half]);
-    dst[i] = from_float<T>(x1 * cs[i] - x2 * sn[i]);
-    dst[i + half] = from_float<T>(x2 * cs[i] + x1 * sn[i]);
-  }
   const int tail = head_dim - rot_dim;  // elements that are not rotated
-  for (int idx = threadIdx.x; idx < kv_heads * tail; idx += blockDim.x) {
-    const int h = idx / tail, i = rot_dim + idx % tail;
-    k_pool[(slot_row + h * head_rows) * head_dim + i] = krow[h * head_dim + i];
+  const int n_pairs = (heads + kv_heads) * half;
+  const int n_tail = (heads + kv_heads) * tail;
+  const int n_values = kv_heads * head_dim;
+  const int item = blockIdx.y * kRopeThreads + threadIdx.x;
+
+  if (item < n_pairs) {
+    const int h = item / half, i = item % half;
+    const int col = h * head_dim + i;
+    const float x1 = in(col), x2 = in(col + half);
+    const float o1 = x1 * cs[i] - x2 * sn[i], o2 = x2 * cs[i] + x1 * sn[i];
+    if (h < heads) {
+      row[col] = from_float<T>(o1);
+      row[col + half] = from_float<T>(o2);
+    } else if (page >= 0) {
+      T* dst = k_pool + page_base + (static_cast<size_t>(h - heads) * page_size + slot) * head_dim;
+      dst[i] = from_float<T>(o1);
+      dst[i + half] = from_float<T>(o2);
+    }
+  } else if (item < n_pairs + n_tail) {
+    const int e = item - n_pairs;
+    const int h = e / tail, i = rot_dim + e % tail;
+    const float x = in(h * head_dim + i);
+    if (h < heads) {
+      row[h * head_dim + i] = from_float<T>(x);
+    } else if (page >= 0) {
+      k_pool[page_base + (static_cast<size_t>(h - heads) * page_size + slot) * head_dim + i] =
+          from_float<T>(x);
+    }
+  } else if (item < n_pairs + n_tail + n_values) {
+    const int e = item - n_pairs - n_tail;  // kv head * head_dim + element
+    if (page >= 0)
+      v_pool[page_base + static_cast<size_t>(e) * page_size + slot] =
+          from_float<T>(in((heads + kv_heads) * head_dim + e));
   }
-  // values: stored transposed, [page][kv head][head_dim][page_size], so that the
-  // keys of a page are contiguous for every element (the operand layout of P.V)
-  const T* vrow = krow + kv_heads * head_dim;
-  const size_t vbase = static_cast<size_t>(page) * kv_heads * head_dim * page_size + pos % page_size;
-  for (int idx = threadIdx.x; idx < kv_heads * head_dim; idx += blockDim.x)
-    v_pool[vbase + static_cast<size_t>(idx) * page_size] = vrow[idx];
 }
 
 }  // namespace shk
@@ -84,6 +105,7 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
                                  const int32_t* positions, const int32_t* token_seq,
                                  const int32_t* tables, int table_stride, void* k_pool,
                                  void* v_pool, int page_size, int num_pages, int write_kv,
+                                 const float* parts, int splits, const float* bias,
                                  void* stream) {
   SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "rope_kv_store: unknown dtype %d", dtype);
   SHK_REQUIRE(n >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0,
@@ -93,7 +115,10 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
               "rope_kv_store: rot_dim %d must be even and at most head_dim %d", rot_dim, head_dim);
   SHK_REQUIRE(rot_dim / 2 <= kMaxHalf, "rope_kv_store: rot_dim %d exceeds %d", rot_dim,
               2 * kMaxHalf);
+  SHK_REQUIRE(splits >= 0 && (splits == 0 || parts), "rope_kv_store: partial sums without a pointer");
   if (n == 0) return 0;
+  SHK_REQUIRE(n <= 2147483647 / ((heads + 2 * kv_heads) * head_dim),
+              "rope_kv_store: too many tokens (%d)", n);
   SHK_REQUIRE(qkv && positions, "rope_kv_store: null pointer");
   SHK_REQUIRE(rot_dim == 0 || inv_freq, "rope_kv_store: rotation needs inv_freq");
   if (write_kv) {
@@ -102,17 +127,20 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
                 "rope_kv_store: bad cache sizes page_size=%d num_pages=%d table_stride=%d",
                 page_size, num_pages, table_stride);
   }
+  const int items = (heads + kv_heads) * (head_dim - rot_dim / 2) + kv_heads * head_dim;
+  dim3 grid(n, (items + kRopeThreads - 1) / kRopeThreads);
+  SHK_REQUIRE(grid.y <= 65535, "rope_kv_store: too many elements per token");
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == kF32)
-    rope_kv_store_kernel<float><<<n, 256, 0, s>>>(
-        static_cast<float*>(qkv), heads, kv_heads, head_dim, rot_dim, inv_freq, positions,
+    rope_kv_store_kernel<float><<<grid, kRopeThreads, 0, s>>>(
+        static_cast<float*>(qkv), n, heads, kv_heads, head_dim, rot_dim, inv_freq, positions,
         token_seq, tables, table_stride, static_cast<float*>(k_pool), static_cast<float*>(v_pool),
-        page_size, num_pages, write_kv);
+        page_size, num_pages, write_kv, parts, splits, bias);
   else
-    rope_kv_store_kernel<bf16><<<n, 256, 0, s>>>(
-        static_cast<bf16*>(qkv), heads, kv_heads, head_dim, rot_dim, inv_freq, positions,
+    rope_kv_store_kernel<bf16><<<grid, kRopeThreads, 0, s>>>(
+        static_cast<bf16*>(qkv), n, heads, kv_heads, head_dim, rot_dim, inv_freq, positions,
         token_seq, tables, table_stride, static_cast<bf16*>(k_pool), static_cast<bf16*>(v_pool),
-        page_size, num_pages, write_kv);
+        page_size, num_pages, write_kv, parts, splits, bias);
   SHK_LAUNCH_CHECK("rope_kv_store");
   return 0;
 }

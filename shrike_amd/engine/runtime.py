@@ -40,12 +40,47 @@ class Runtime:
             return LinearWeight(w.shape, None, ops.retile_weight(w))
         return LinearWeight(w.shape, w, None)
 
+    def gated_weight(self, gate: torch.Tensor, up: torch.Tensor):
+        """The two matrices of a gated feed-forward, as `gated_linear` wants them."""
+        if self.dtype == torch.bfloat16:
+            tiled = ops.interleave_gate_up(gate.contiguous(), up.contiguous())
+            return LinearWeight(gate.shape, None, tiled)
+        return self.weight(torch.cat([gate, up], dim=0))
+
+    def gated_linear(self, ctx, x, w: LinearWeight, out) -> None:
+        """out = silu(x @ gate.T) * (x @ up.T).  bfloat16: one product whose
+        epilogue applies the activation; float32: product, then activation."""
+        if w.tiled is not None:
+            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, gated=True)
+            return
+        gate_up = ctx.buffer("ffn_gate_up", (x.shape[0], w.rows), self.dtype)
+        ops.gemm(x, w.dense, gate_up)
+        ops.silu_mul(gate_up, out)
+
     def linear(self, x, w: LinearWeight, out, bias=None, accumulate=False) -> None:
         """out (+)= x @ w.T + bias."""
         if w.tiled is not None:
             ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, bias=bias, accumulate=accumulate)
         else:
             ops.gemm(x, w.dense, out, bias=bias, accumulate=accumulate)
+
+    def linear_deferred(self, ctx, name: str, x, w: LinearWeight, bias=None, reader="norm"):
+        """x @ w.T + bias for a reader that can add up partial sums: a tensor
+        [n, rows] in the compute dtype, or, where a matrix with few rows is split
+        along k to fill the chip, the SplitSum of its parts.  reader "norm": the
+        residual add of the next norm (no bias, width a multiple of 4 up to
+        8192); reader "position": the position-encoding and cache-write kernel."""
+        n = x.shape[0]
+        splits = ops.gemm_splits(n, w.rows, w.cols) if w.tiled is not None else 1
+        if reader == "norm" and (bias is not None or w.rows % 4 or w.rows > 8192):
+            splits = 1
+        if splits > 1:
+            parts = ctx.buffer(name + "_parts", (splits, n, w.rows), torch.float32)
+            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, parts, splits=splits)
+            return ops.SplitSum(parts, bias)
+        out = ctx.buffer(name, (n, w.rows), self.dtype)
+        self.linear(x, w, out, bias=bias)
+        return out
 
     def attend(self, ctx, qkv, out, spec, tables, cache) -> None:
         """Attention of every token of the step over its sequence's cache."""

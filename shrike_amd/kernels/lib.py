@@ -18,12 +18,14 @@ _P, _I, _F = c_void_p, c_int, c_float
 
 _SIGNATURES = {
     "shk_embed": [_P, _I, _P, _P, _I, _I, _I, _P],
-    "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _P],
+    "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "shk_silu_mul": [_P, _P, _I, _I, _I, _P],
     "shk_gemm": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "shk_retile_weight": [_P, _I, _I, _P, _P],
-    "shk_gemm_bf16_tiled_weight": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-    "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P],
+    "shk_interleave_gate_up": [_P, _P, _I, _I, _P, _P],
+    "shk_gemm_bf16_tiled_weight": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "shk_gemm_bf16_splits": [_I, _I, _I],
+    "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _P],
     "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _P],
     "shk_attention_supports_mfma": [_I, _I, _I, _I, _I],
     "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _P, _I, _P],

@@ -36,6 +36,22 @@ def _rows(t: torch.Tensor, name: str) -> None:
         raise KernelError(f"{name}: expected a 2-d tensor with unit inner stride")
 
 
+class SplitSum:
+    """The float32 partial sums [splits, n, m] of a product that was split
+    along k, with the bias that is still to be added.  Kernels that read the
+    product (add_rmsnorm, rope_kv_store) add the parts up in order."""
+
+    __slots__ = ("parts", "bias")
+
+    def __init__(self, parts: torch.Tensor, bias: torch.Tensor | None = None):
+        self.parts = parts
+        self.bias = bias
+
+    @property
+    def shape(self):
+        return self.parts.shape[1:]
+
+
 def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
     """out[i] = float(table[ids[i]]); ids int32 [n], out float32 [n, hidden]."""
     n, hidden = out.shape
@@ -55,7 +71,14 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_resid=Tr
     n, hidden = out.shape
     if not (resid.is_contiguous() and out.is_contiguous() and resid.shape[1] == hidden):
         raise KernelError("add_rmsnorm: resid/out must be contiguous with the same width")
-    if delta is not None and (
+    splits = 0
+    if isinstance(delta, SplitSum):
+        if delta.bias is not None or tuple(delta.shape) != tuple(resid.shape):
+            raise KernelError("add_rmsnorm: partial sums must match resid's shape and carry no bias")
+        splits, delta = delta.parts.shape[0], delta.parts
+        if delta.dtype != torch.float32 or not delta.is_contiguous():
+            raise KernelError("add_rmsnorm: partial sums must be contiguous float32")
+    elif delta is not None and (
         delta.dtype != out.dtype or not delta.is_contiguous() or delta.shape != resid.shape
     ):
         raise KernelError("add_rmsnorm: delta must match resid's shape and out's dtype")
@@ -69,7 +92,7 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_resid=Tr
             None if delta is None else _dev(delta, "delta"),
             _dev(weight, "weight", torch.float32), float(eps), _dev(out, "out"),
             dtype_code(out.dtype), None if rows is None else _dev(rows, "rows", torch.int32),
-            n, hidden, int(bool(write_resid)), _stream(),
+            n, hidden, int(bool(write_resid)), splits, resid.shape[0], _stream(),
         )
     )
 
@@ -124,17 +147,41 @@ def retile_weight(w: torch.Tensor) -> torch.Tensor:
     return wt
 
 
-def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False) -> None:
+def interleave_gate_up(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """The tiled layouts of two row-major [m, k] matrices interleaved by blocks of
+    16 rows, for the gated product of gemm_tiled_weight."""
+    if gate.shape != up.shape:
+        raise KernelError("interleave_gate_up: gate and up differ in shape")
+    m, k = gate.shape
+    gt, ut = retile_weight(gate), retile_weight(up)
+    wt = torch.empty(2 * tiled_numel(m, k), dtype=torch.bfloat16, device=gate.device)
+    check(load().shk_interleave_gate_up(_dev(gt, "gate"), _dev(ut, "up"), m, k, _dev(wt, "wt"),
+                                        _stream()))
+    return wt
+
+
+def gemm_splits(n: int, m: int, k: int) -> int:
+    """Shares of k that fill the chip for an [n, k] x [m, k]^T product (1: do not split)."""
+    return int(load().shk_gemm_bf16_splits(n, m, k))
+
+
+def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, gated=False,
+                      splits: int = 1) -> None:
     """out (+)= a @ w.T + bias with wt = retile_weight(w): up to 64 rows of a
-    stream the weights once; more rows run the LDS-staged MFMA kernel."""
+    stream the weights once; more rows run the LDS-staged MFMA kernel.
+    splits > 1: out is float32 [splits, n, m] and receives partial sums."""
     _rows(a, "gemm a")
-    _rows(out, "gemm out")
     n = a.shape[0]
     if a.shape[1] != k or a.dtype != torch.bfloat16:
         raise KernelError(f"gemm_tiled_weight: a must be bfloat16 [n, {k}], got {tuple(a.shape)}")
-    if out.shape != (n, m):
-        raise KernelError(f"gemm_tiled_weight: out must be [{n}, {m}], got {tuple(out.shape)}")
-    if wt.numel() != tiled_numel(m, k) or wt.dtype != torch.bfloat16:
+    if splits > 1:
+        if tuple(out.shape) != (splits, n, m) or not out.is_contiguous() or out.dtype != torch.float32:
+            raise KernelError(f"gemm_tiled_weight: partial sums must be contiguous float32 [{splits}, {n}, {m}]")
+    else:
+        _rows(out, "gemm out")
+        if out.shape != (n, m):
+            raise KernelError(f"gemm_tiled_weight: out must be [{n}, {m}], got {tuple(out.shape)}")
+    if wt.numel() != (2 if gated else 1) * tiled_numel(m, k) or wt.dtype != torch.bfloat16:
         raise KernelError("gemm_tiled_weight: wt is not the tiled layout of an [m, k] matrix")
     if bias is not None and bias.numel() != m:
         raise KernelError(f"gemm_tiled_weight: bias has {bias.numel()} elements, m is {m}")
@@ -142,8 +189,8 @@ def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False) -
         load().shk_gemm_bf16_tiled_weight(
             _dev(a, "a"), _dev(wt, "wt"),
             None if bias is None else _dev(bias, "bias", torch.float32),
-            _dev(out, "out"), n, m, k, a.stride(0), out.stride(0), dtype_code(out.dtype),
-            int(bool(accumulate)), _stream(),
+            _dev(out, "out"), n, m, k, a.stride(0), out.stride(-2), dtype_code(out.dtype),
+            int(bool(accumulate)), int(bool(gated)), int(splits), _stream(),
         )
     )
 
@@ -167,13 +214,19 @@ def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size) 
 
 
 def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, token_seq,
-                  tables, k_pool, v_pool, page_size, write_kv=True) -> None:
+                  tables, k_pool, v_pool, page_size, write_kv=True, split_sum=None) -> None:
     """Rotate q and k of qkv [n, (heads + 2 kv_heads) head_dim] in float32 and put
     k, v into their pages (keys [pages, kv_heads, page_size, head_dim], values
     transposed [pages, kv_heads, head_dim, page_size])."""
     n = qkv.shape[0]
     if not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
         raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim]")
+    parts, splits, bias = None, 0, None
+    if split_sum is not None:
+        parts, bias = split_sum.parts, split_sum.bias
+        splits = parts.shape[0]
+        if tuple(parts.shape[1:]) != tuple(qkv.shape) or parts.dtype != torch.float32 or not parts.is_contiguous():
+            raise KernelError("rope_kv_store: partial sums must be contiguous float32 [splits, n, width]")
     num_pages = 0
     if write_kv:
         _check_pools("rope_kv_store", qkv, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
@@ -188,7 +241,9 @@ def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, 
             tables.shape[1] if write_kv else 0,
             _dev(k_pool, "k_pool") if write_kv else None,
             _dev(v_pool, "v_pool") if write_kv else None,
-            page_size, num_pages, int(bool(write_kv)), _stream(),
+            page_size, num_pages, int(bool(write_kv)),
+            None if parts is None else _dev(parts, "parts", torch.float32), splits,
+            None if bias is None else _dev(bias, "bias", torch.float32), _stream(),
         )
     )
 

@@ -76,30 +76,37 @@ class PagedAttention(Mixer):
         if self.position is not None:
             self.position.load(tensors, runtime)
         self.linear = runtime.linear
+        self.linear_deferred = runtime.linear_deferred
         self.attend = runtime.attend
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
         s = self.spec
         n = x.shape[0]
         qkv_width = (s.num_heads + 2 * s.num_kv_heads) * s.head_dim
-        qkv = ctx.buffer("attn_qkv", (n, qkv_width), ctx.dtype)
-        self.linear(x, self.w_qkv, qkv, bias=self.b_qkv)
-
         table = self.position.rotary_table() if self.position is not None else None
-        if self.position is not None and table is None:
+        fused_position = self.position is None or table is not None
+        split_sum = None
+        if fused_position:
+            # the cache-write kernel can take the projections as partial sums
+            qkv = self.linear_deferred(ctx, "attn_qkv_sum", x, self.w_qkv, bias=self.b_qkv,
+                                       reader="position")
+            if isinstance(qkv, ops.SplitSum):
+                split_sum, qkv = qkv, ctx.buffer("attn_qkv", (n, qkv_width), ctx.dtype)
+        else:
+            qkv = ctx.buffer("attn_qkv", (n, qkv_width), ctx.dtype)
+            self.linear(x, self.w_qkv, qkv, bias=self.b_qkv)
             self.position.apply(ctx, qkv, s.num_heads, s.num_kv_heads, s.head_dim)
         inv_freq, rot_dim = table if table is not None else (None, 0)
         tables = ctx.block_tables[cache.group]
         ops.rope_kv_store(
             qkv, s.num_heads, s.num_kv_heads, s.head_dim, rot_dim, inv_freq, ctx.positions,
             ctx.token_seq, tables, cache.k_pool, cache.v_pool, cache.page_size,
-            write_kv=cache.owned,
+            write_kv=cache.owned, split_sum=split_sum,
         )
         attn = ctx.buffer("attn_out", (n, s.num_heads * s.head_dim), ctx.dtype)
         self.attend(ctx, qkv, attn, s, tables, cache)
-        out = ctx.buffer("attn_proj", (n, self.width), ctx.dtype)
-        self.linear(attn, self.w_o, out, bias=self.b_o)
-        return out
+        # the norm that follows adds the output to the residual stream and can add up parts
+        return self.linear_deferred(ctx, "attn_proj", attn, self.w_o, bias=self.b_o)
 
 
 register_mixer("paged_attention", PagedAttention)

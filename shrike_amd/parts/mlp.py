@@ -4,14 +4,13 @@ from __future__ import annotations
 
 import torch
 
-from ..kernels import ops
 from .base import FeedForward, ParamSpec, register_ffn
 
 
 class SwiGLU(FeedForward):
     """down(silu(gate(x)) * up(x)) without biases (reference:
-    shrike/models/qwen.py:131-136).  gate and up are stacked into one [2I, h]
-    matrix at load time so that one product feeds the activation kernel."""
+    shrike/models/qwen.py:131-136).  gate and up are joined into one weight at
+    load time, so that one product yields the activated values."""
 
     def params(self):
         inter, h = self.spec.intermediate_size, self.width
@@ -23,21 +22,19 @@ class SwiGLU(FeedForward):
 
     def load(self, tensors, runtime):
         self.inter = int(self.spec.intermediate_size)
-        self.w_gate_up = runtime.weight(torch.cat(
-            [tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]], dim=0
-        ))
+        self.w_gate_up = runtime.gated_weight(
+            tensors[f"{self.name}.gate_proj.weight"], tensors[f"{self.name}.up_proj.weight"]
+        )
         self.w_down = runtime.weight(tensors[f"{self.name}.down_proj.weight"])
-        self.linear = runtime.linear
+        self.linear_deferred = runtime.linear_deferred
+        self.gated_linear = runtime.gated_linear
 
     def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
         n = x.shape[0]
-        gate_up = ctx.buffer("ffn_gate_up", (n, 2 * self.inter), ctx.dtype)
-        self.linear(x, self.w_gate_up, gate_up)
         act = ctx.buffer("ffn_act", (n, self.inter), ctx.dtype)
-        ops.silu_mul(gate_up, act)
-        out = ctx.buffer("ffn_out", (n, self.width), ctx.dtype)
-        self.linear(act, self.w_down, out)
-        return out
+        self.gated_linear(ctx, x, self.w_gate_up, act)
+        # the norm that follows adds the output to the residual stream and can add up parts
+        return self.linear_deferred(ctx, "ffn_out", act, self.w_down)
 
 
 register_ffn("swiglu", SwiGLU)

@@ -370,7 +370,7 @@ def test_sample_frequencies_follow_the_distribution(ops):
     "n, m, k",
     [(1, 48, 64), (8, 3584, 3584), (7, 503, 128), (16, 100, 172), (17, 130, 96), (33, 200, 333),
      (48, 64, 64), (64, 1000, 520), (5, 37, 50), (65, 128, 64), (130, 200, 333), (300, 503, 128),
-     (1000, 172, 96), (257, 130, 172), (2048, 1024, 512)],
+     (1000, 172, 96), (257, 130, 172), (2048, 1024, 512), (33, 200, 1600), (3, 48, 4000), (64, 100, 2100)],
 )
 def test_gemm_tiled_weight(ops, n, m, k):
     """The MFMA kernels over the tiled weight layout (weight-streaming up to 64
@@ -502,3 +502,79 @@ def test_attention_mfma_finds_one_far_key_among_thousands(ops):
     assert torch.allclose(got[3], v[far, 0].to(dtype).float(), atol=3e-2)
     want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, [1], [ctx - 1], page_size, None, 1.0)
     close(out.view(1, heads, head_dim), want, dtype, scale=1.0)
+
+
+@pytest.mark.parametrize("n, inter, k", [(1, 172, 64), (8, 18944, 256), (20, 100, 96), (40, 352, 128), (64, 48, 50),
+                                         (9, 100, 1700), (50, 64, 3000),
+                                         (65, 172, 64), (300, 1000, 520), (1000, 200, 96)])
+def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
+    """One product over the interleaved gate/up weight yields silu(x g^T) * (x u^T)."""
+    torch.manual_seed(17)
+    dtype = torch.bfloat16
+    x = torch.randn(n, k)
+    g, u = torch.randn(inter, k) / math.sqrt(k) * 2, torch.randn(inter, k) / math.sqrt(k)
+    wt = ops.interleave_gate_up(dev(g, dtype), dev(u, dtype))
+    out = torch.full((n, inter), float("nan"), device="cuda", dtype=dtype)
+    ops.gemm_tiled_weight(dev(x, dtype), wt, inter, k, out, gated=True)
+    gate = rounded(x, dtype) @ rounded(g, dtype).t()
+    want = gate * torch.sigmoid(gate) * (rounded(x, dtype) @ rounded(u, dtype).t())
+    close(out, want, dtype)
+
+
+@pytest.mark.parametrize("n, m, k", [(8, 3584, 3584), (1, 48, 4000), (33, 200, 1600), (64, 100, 2100)])
+def test_split_product_and_its_readers(ops, n, m, k):
+    """A product split along k leaves partial sums; the norm and the cache-write
+    kernel add them up in order and give what the unsplit product gives."""
+    torch.manual_seed(18)
+    dtype = torch.bfloat16
+    splits = ops.gemm_splits(n, m, k)
+    assert splits > 1 and ops.gemm_splits(n, 20000, k) == 1 and ops.gemm_splits(100, m, k) == 1
+    a, w = torch.randn(n, k), torch.randn(m, k) / math.sqrt(k)
+    wt = ops.retile_weight(dev(w, dtype))
+    parts = torch.full((splits, n, m), float("nan"), device="cuda")
+    ops.gemm_tiled_weight(dev(a, dtype), wt, m, k, parts, splits=splits)
+    want = rounded(a, dtype) @ rounded(w, dtype).t()
+    close(parts.sum(0), want, torch.float32, scale=want.abs().max() * 50)
+    total = parts[0].clone()
+    for z in range(1, splits):
+        total += parts[z]
+    # the norm adds the parts to the residual stream
+    if m % 4 == 0:
+        resid = torch.randn(n, m, device="cuda")
+        before = resid.clone()
+        wn = 1 + 0.1 * torch.randn(m, device="cuda")
+        out = torch.empty(n, m, device="cuda", dtype=dtype)
+        ops.add_rmsnorm(resid, ops.SplitSum(parts), wn, 1e-5, out)
+        assert torch.equal(resid, before + total)
+        close(out, plain.rms_norm((before + total).double().cpu(), wn.double().cpu(), 1e-5), dtype)
+
+
+def test_rope_kv_store_adds_up_a_split_product(ops):
+    torch.manual_seed(19)
+    dtype = torch.bfloat16
+    heads, kv_heads, head_dim, page_size, theta = 6, 2, 64, 16, 1e4
+    n, splits = 5, 3
+    width = (heads + 2 * kv_heads) * head_dim
+    parts = torch.randn(splits, n, width, device="cuda")
+    bias = torch.randn(width, device="cuda")
+    positions = torch.tensor([3, 17, 100, 0, 31], dtype=torch.int32, device="cuda")
+    token_seq = torch.arange(n, dtype=torch.int32, device="cuda")
+    tables, k_pool, v_pool = paged_setup([p + 1 for p in positions.tolist()], page_size, 32, kv_heads, head_dim, dtype)
+    inv_freq = (1.0 / (theta ** (torch.arange(0, head_dim, 2).float() / head_dim))).cuda()
+    qkv = torch.full((n, width), float("nan"), device="cuda", dtype=dtype)
+    ops.rope_kv_store(qkv, heads, kv_heads, head_dim, head_dim, inv_freq, positions, token_seq, tables,
+                      k_pool, v_pool, page_size, split_sum=ops.SplitSum(parts, bias))
+    total = parts[0].clone()
+    for z in range(1, splits):
+        total += parts[z]
+    x = (total + bias).double().cpu()
+    cos, sin = plain.rope_tables(positions.long().cpu(), head_dim, theta)
+    q = plain.apply_rope(x[:, : heads * head_dim].view(n, heads, head_dim), cos, sin)
+    close(qkv[:, : heads * head_dim].reshape(n, heads, head_dim), q, dtype)
+    k = plain.apply_rope(x[:, heads * head_dim : (heads + kv_heads) * head_dim].view(n, kv_heads, head_dim), cos, sin)
+    v = x[:, (heads + kv_heads) * head_dim :].view(n, kv_heads, head_dim)
+    for t in range(n):
+        p = int(positions[t])
+        page = int(tables[t, p // page_size])
+        close(k_pool[page, :, p % page_size], k[t], dtype)
+        close(v_pool[page, :, :, p % page_size], v[t], dtype)
