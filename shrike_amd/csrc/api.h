@@ -115,8 +115,12 @@ int shk_attention_prefill_bf16(const void* q, int q_stride, void* out, int num_t
                                const void* k_pool, const void* v_pool, int page_size, int window,
                                float scale, void* stream);
 
-// out[r] = lowest index of the largest value of logits[r, :vocab].
-int shk_argmax(const float* logits, int32_t* out, int rows, int vocab, int ld, void* stream);
+// out[r] = lowest index of the largest value of logits[r, :vocab].  Rows wider
+// than 4096 are searched in chunks; scratch then holds
+// shk_argmax_scratch_floats(rows, vocab) floats (0: not needed).
+int shk_argmax(const float* logits, int32_t* out, int rows, int vocab, int ld, float* scratch,
+               void* stream);
+int shk_argmax_scratch_floats(int rows, int vocab);
 
 // Temperature / top-p sampling of one token per row (see sampling.hip).
 // temperature[r] == 0 takes the argmax.  uniforms[r] in [0, 1) is the draw.

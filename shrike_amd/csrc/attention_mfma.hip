@@ -33,6 +33,27 @@ union AFrag {
 
 constexpr int kPStride = 40;  // bf16 elements per row of the P tile in LDS (32 + padding)
 
+// A window of 64 entries of a sequence's block table held across the lanes of
+// the wavefront (lane i: entry base + i), so that finding a key's page is a
+// register exchange instead of a load that the key and value loads wait for.
+struct PageWindow {
+  int base;     // index of the first entry held
+  int32_t mine;  // this lane's entry
+};
+
+__device__ __forceinline__ PageWindow load_pages(const int32_t* table, int first, int last) {
+  // entries first .. first + 63, none beyond `last` (the last entry the keys reach)
+  PageWindow w;
+  w.base = first;
+  const int i = first + static_cast<int>(threadIdx.x % kWave);
+  w.mine = (i <= last) ? table[i] : 0;
+  return w;
+}
+
+__device__ __forceinline__ int page_at(const PageWindow& w, int entry) {
+  return __shfl(w.mine, entry - w.base, kWave);
+}
+
 struct TileArgs {
   const int32_t* table;  // block table of the sequence
   const bf16* k_pool;    // [pages][kv_heads][page_size][D]
@@ -54,8 +75,8 @@ struct Chunk {
 // Issues every load of the chunk at key `kb`; tiles and key groups that no row
 // reads (beyond pos_max, before lo_min) are not touched and read as zero.
 template <int D>
-__device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, int kb, int pos_max,
-                                           int lo_min) {
+__device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, const PageWindow& pw,
+                                           int kb, int pos_max, int lo_min) {
   const int lane = threadIdx.x % kWave;
   const int j = lane % 16, kg = lane / 16;
   const int ps = ta.page_size;
@@ -65,8 +86,9 @@ __device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, int 
     const int key0 = kb + tt * 16;
     const bool live = key0 <= pos_max && key0 + 15 >= lo_min;
     const bf16* krow = nullptr;
+    const int kpage = page_at(pw, (key0 <= pos_max ? key0 : pos_max) / ps);
     if (live) {
-      const int page = ta.table[key0 / ps];
+      const int page = kpage;
       krow = ta.k_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
              static_cast<size_t>(key0 % ps + j) * D + kg * 8;
     }
@@ -80,8 +102,9 @@ __device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, int 
   const int g0 = kb + kg * 8;
   const bool live = g0 <= pos_max && g0 + 7 >= lo_min;
   const bf16* vcol = nullptr;
+  const int vpage = page_at(pw, (g0 <= pos_max ? g0 : pos_max) / ps);
   if (live) {
-    const int page = ta.table[g0 / ps];
+    const int page = vpage;
     vcol = ta.v_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
            static_cast<size_t>(j) * ps + g0 % ps;
   }
@@ -106,10 +129,17 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
   const int lane = threadIdx.x % kWave;
   const int j = lane % 16, kg = lane / 16;
 
+  const int ps = ta.page_size;
+  const int last_entry = pos_max / ps;
+  PageWindow pw = load_pages(ta.table, key_begin / ps, last_entry);
   Chunk<D> cur, nxt;
-  if (key_begin < key_end) load_chunk<D>(cur, ta, key_begin, pos_max, lo_min);
+  if (key_begin < key_end) load_chunk<D>(cur, ta, pw, key_begin, pos_max, lo_min);
   for (int kb = key_begin; kb < key_end; kb += 32) {
-    if (kb + 32 < key_end) load_chunk<D>(nxt, ta, kb + 32, pos_max, lo_min);
+    if (kb + 32 < key_end) {
+      // the window must hold the entries of keys kb + 32 .. kb + 63
+      if ((kb + 63) / ps >= pw.base + kWave) pw = load_pages(ta.table, (kb + 32) / ps, last_entry);
+      load_chunk<D>(nxt, ta, pw, kb + 32, pos_max, lo_min);
+    }
 
     // ---- S = Q K^T for two tiles of 16 keys
     f32x4 s[2];

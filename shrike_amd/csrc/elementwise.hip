@@ -30,12 +30,12 @@ __global__ void embed_kernel(const T* __restrict__ table, const int32_t* __restr
 
 // ------------------------------------------------------------ add + RMSNorm
 // One workgroup per row.  add_rmsnorm_vec_kernel holds the row in registers
-// (hidden a multiple of 4, at most 256 * 4 * kNormVecs elements): all loads
-// are issued before the first use, so a row costs one memory round trip.
+// (hidden a multiple of 4, at most 8192 elements): all loads are issued
+// before the first use, so a row costs one memory round trip.
 // add_rmsnorm_kernel takes every other size.
 
 constexpr int kNormThreads = 256;
-constexpr int kNormVecs = 8;  // float4 per thread: rows of up to 8192 elements
+constexpr int kNormVecs = 2;  // float4 per thread: rows of up to 8192 elements with 1024 threads
 
 __device__ __forceinline__ float4 load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 __device__ __forceinline__ float4 load4(const bf16* p) {
@@ -52,9 +52,10 @@ __device__ __forceinline__ void store4(bf16* p, float4 v) {
 }
 
 // TD is the type of delta: T, or float for the partial sums of a split product
-// ([splits][resid_rows][hidden], added in order).
-template <typename T, typename TD>
-__global__ void __launch_bounds__(kNormThreads)
+// ([splits][resid_rows][hidden], added in order).  THREADS * 4 * kNormVecs
+// elements fit; wide rows get 1024 threads so that few loads follow each other.
+template <typename T, typename TD, int THREADS>
+__global__ void __launch_bounds__(THREADS)
     add_rmsnorm_vec_kernel(float* __restrict__ resid, const TD* __restrict__ delta,
                            const float* __restrict__ weight, float eps, T* __restrict__ out,
                            const int32_t* __restrict__ rows, int hidden, int write_resid,
@@ -70,7 +71,7 @@ __global__ void __launch_bounds__(kNormThreads)
   float4 v[kNormVecs], dv[kNormVecs], w[kNormVecs];
 #pragma unroll
   for (int i = 0; i < kNormVecs; ++i) {
-    const int c = threadIdx.x + i * kNormThreads;
+    const int c = threadIdx.x + i * THREADS;
     v[i] = dv[i] = w[i] = make_float4(0.f, 0.f, 0.f, 0.f);
     if (c < nvec) {
       v[i] = load4(x + c * 4);
@@ -78,17 +79,23 @@ __global__ void __launch_bounds__(kNormThreads)
       w[i] = load4(weight + c * 4);
     }
   }
-  for (int z = 1; z < splits; ++z) {
-    float4 more[kNormVecs];
+  // further parts, four at a time in flight, added in order
+  for (int z0 = 1; z0 < splits; z0 += 4) {
+    float4 more[4][kNormVecs];
 #pragma unroll
-    for (int i = 0; i < kNormVecs; ++i) {
-      const int c = threadIdx.x + i * kNormThreads;
-      more[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (c < nvec) more[i] = load4(d + z * split_stride + c * 4);
-    }
+    for (int u = 0; u < 4; ++u)
 #pragma unroll
-    for (int i = 0; i < kNormVecs; ++i)
-      dv[i].x += more[i].x, dv[i].y += more[i].y, dv[i].z += more[i].z, dv[i].w += more[i].w;
+      for (int i = 0; i < kNormVecs; ++i) {
+        const int c = threadIdx.x + i * THREADS;
+        more[u][i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (c < nvec && z0 + u < splits) more[u][i] = load4(d + (z0 + u) * split_stride + c * 4);
+      }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int i = 0; i < kNormVecs; ++i)
+        dv[i].x += more[u][i].x, dv[i].y += more[u][i].y, dv[i].z += more[u][i].z,
+            dv[i].w += more[u][i].w;
   }
   float ss = 0.f;
 #pragma unroll
@@ -100,7 +107,7 @@ __global__ void __launch_bounds__(kNormThreads)
   const float inv = rsqrtf(ss / static_cast<float>(hidden) + eps);
 #pragma unroll
   for (int i = 0; i < kNormVecs; ++i) {
-    const int c = threadIdx.x + i * kNormThreads;
+    const int c = threadIdx.x + i * THREADS;
     if (c >= nvec) continue;
     if (d && write_resid) store4(x + c * 4, v[i]);
     store4(y + c * 4, make_float4((v[i].x * inv) * w[i].x, (v[i].y * inv) * w[i].y,
@@ -185,34 +192,40 @@ extern "C" int shk_add_rmsnorm(float* resid, const void* delta, const float* wei
   SHK_REQUIRE(resid && weight && out, "add_rmsnorm: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  const bool vec = hidden % 4 == 0 && hidden <= kNormThreads * 4 * kNormVecs && aligned(resid) &&
+  const bool vec = hidden % 4 == 0 && hidden <= 1024 * 4 * kNormVecs && aligned(resid) &&
                    aligned(weight) && aligned(out) && (!delta || aligned(delta));
+  SHK_REQUIRE(delta_splits == 0 || (delta && vec && dtype == kBF16 && resid_rows > 0),
+              "add_rmsnorm: partial sums need bfloat16 output, hidden %% 4 == 0 and at most 8192");
+  const size_t stride = static_cast<size_t>(resid_rows) * hidden;
+  const int splits = delta_splits > 0 ? delta_splits : 1;
+#define SHK_NORM(T, TD, THREADS)                                                              \
+  add_rmsnorm_vec_kernel<T, TD, THREADS><<<n, THREADS, 0, s>>>(                               \
+      resid, static_cast<const TD*>(delta), weight, eps, static_cast<T*>(out), rows, hidden,  \
+      write_resid, splits, stride)
+#define SHK_NORM_T(T, TD)                \
+  do {                                   \
+    if (hidden <= 256 * 4 * kNormVecs)   \
+      SHK_NORM(T, TD, 256);              \
+    else                                 \
+      SHK_NORM(T, TD, 1024);             \
+  } while (0)
   if (delta_splits > 0) {
-    SHK_REQUIRE(delta && vec && dtype == kBF16 && resid_rows > 0,
-                "add_rmsnorm: partial sums need bfloat16 output, hidden %% 4 == 0 and at most %d",
-                kNormThreads * 4 * kNormVecs);
-    add_rmsnorm_vec_kernel<bf16, float><<<n, kNormThreads, 0, s>>>(
-        resid, static_cast<const float*>(delta), weight, eps, static_cast<bf16*>(out), rows, hidden,
-        write_resid, delta_splits, static_cast<size_t>(resid_rows) * hidden);
+    SHK_NORM_T(bf16, float);
+  } else if (vec && dtype == kF32) {
+    SHK_NORM_T(float, float);
+  } else if (vec) {
+    SHK_NORM_T(bf16, bf16);
   } else if (dtype == kF32) {
-    if (vec)
-      add_rmsnorm_vec_kernel<float, float><<<n, kNormThreads, 0, s>>>(
-          resid, static_cast<const float*>(delta), weight, eps, static_cast<float*>(out), rows,
-          hidden, write_resid, 1, 0);
-    else
-      add_rmsnorm_kernel<float><<<n, kNormThreads, 0, s>>>(
-          resid, static_cast<const float*>(delta), weight, eps, static_cast<float*>(out), rows,
-          hidden, write_resid);
+    add_rmsnorm_kernel<float><<<n, kNormThreads, 0, s>>>(
+        resid, static_cast<const float*>(delta), weight, eps, static_cast<float*>(out), rows,
+        hidden, write_resid);
   } else {
-    if (vec)
-      add_rmsnorm_vec_kernel<bf16, bf16><<<n, kNormThreads, 0, s>>>(
-          resid, static_cast<const bf16*>(delta), weight, eps, static_cast<bf16*>(out), rows,
-          hidden, write_resid, 1, 0);
-    else
-      add_rmsnorm_kernel<bf16><<<n, kNormThreads, 0, s>>>(
-          resid, static_cast<const bf16*>(delta), weight, eps, static_cast<bf16*>(out), rows,
-          hidden, write_resid);
+    add_rmsnorm_kernel<bf16><<<n, kNormThreads, 0, s>>>(
+        resid, static_cast<const bf16*>(delta), weight, eps, static_cast<bf16*>(out), rows, hidden,
+        write_resid);
   }
+#undef SHK_NORM_T
+#undef SHK_NORM
   SHK_LAUNCH_CHECK("add_rmsnorm");
   return 0;
 }

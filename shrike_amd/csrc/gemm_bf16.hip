@@ -175,6 +175,157 @@ __global__ void __launch_bounds__(WAVES* kWave)
   }
 }
 
+// gemm_mid_kernel: for 17 to 64 tokens.  The skinny kernel would fetch the
+// activations once per block of 16 weight rows, which at this many tokens is
+// several times the weight traffic.  Here a workgroup of WAVES wavefronts owns
+// WAVES blocks of weight rows (one per wavefront; a gate and an up block when
+// GATED) and walks k in stages of 128: the stage's activations are staged once
+// in LDS in operand layout and shared by all wavefronts, while each wavefront
+// streams its own weight tiles straight into registers (nobody else needs
+// them).  Both are double-buffered.  ksplit > 1 shares k among workgroups,
+// which leave float32 partial sums [ksplit][n][m] for the reading kernel.
+constexpr int kMidTiles = 4;  // k-tiles per stage
+
+template <int NB, int WAVES, bool GATED>
+__global__ void __launch_bounds__(WAVES* kWave)
+    gemm_mid_kernel(const bf16* __restrict__ a, int lda, int n, int k,
+                    const uint4* __restrict__ wt, int ktiles, int m,
+                    const float* __restrict__ bias, void* __restrict__ out, int ldo, int out_f32,
+                    int accumulate, int vec, int ksplit) {
+  constexpr int RB = GATED ? 2 : 1;
+  __shared__ uint4 act[2][NB][kMidTiles][kWave];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int j = lane % 16, kg = lane / 16;
+  const int ob = blockIdx.x * WAVES + wave;  // block of 16 output rows of this wavefront
+  const int oblocks = (m + 15) / 16;
+  const bool have_rows = ob < oblocks;
+  const uint4* wrow = wt + static_cast<size_t>(have_rows ? ob : 0) * RB * ktiles * kWave + lane;
+
+  const int nstages = (ktiles + kMidTiles - 1) / kMidTiles;
+  const int per = (nstages + ksplit - 1) / ksplit;
+  const int st_begin = blockIdx.y * per;
+  const int st_end = st_begin + per < nstages ? st_begin + per : nstages;
+
+  f32x4 acc[RB][NB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[rb][b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int kItems = NB * kMidTiles * kWave;           // activation fragments-lanes per stage
+  constexpr int kPerThread = (kItems + WAVES * kWave - 1) / (WAVES * kWave);
+  Frag wcur[RB][kMidTiles], wnext[RB][kMidTiles];
+  uint4 areg[kPerThread];
+
+  auto load_weights = [&](Frag (&w)[RB][kMidTiles], int st) {
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int t = 0; t < kMidTiles; ++t) {
+        const int tt = st * kMidTiles + t;
+        w[rb][t].u = make_uint4(0, 0, 0, 0);
+        if (have_rows && tt < ktiles) {
+          const uint4* p = wrow + (static_cast<size_t>(rb) * ktiles + tt) * kWave;
+          w[rb][t].u.x = __builtin_nontemporal_load(&p->x);
+          w[rb][t].u.y = __builtin_nontemporal_load(&p->y);
+          w[rb][t].u.z = __builtin_nontemporal_load(&p->z);
+          w[rb][t].u.w = __builtin_nontemporal_load(&p->w);
+        }
+      }
+  };
+  auto load_acts = [&](int st) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int item = tid + i * WAVES * kWave;  // (b * kMidTiles + t) * 64 + lane
+      areg[i] = make_uint4(0, 0, 0, 0);
+      if (item < kItems) {
+        const int ln = item % kWave, f = item / kWave, t = f % kMidTiles, b = f / kMidTiles;
+        areg[i] = load_act(a, lda, n, k, b * 16 + ln % 16, (st * kMidTiles + t) * 32 + (ln / 16) * 8,
+                           vec).u;
+      }
+    }
+  };
+  auto store_acts = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int item = tid + i * WAVES * kWave;
+      if (item < kItems) (&act[buf][0][0][0])[item] = areg[i];
+    }
+  };
+
+  if (st_begin < st_end) {
+    load_weights(wcur, st_begin);
+    load_acts(st_begin);
+    store_acts(0);
+  }
+  __syncthreads();
+  for (int st = st_begin; st < st_end; ++st) {
+    const int buf = (st - st_begin) & 1;
+    const bool more = st + 1 < st_end;
+    if (more) {
+      load_weights(wnext, st + 1);
+      load_acts(st + 1);
+    }
+#pragma unroll
+    for (int t = 0; t < kMidTiles; ++t)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        Frag x;
+        x.u = act[buf][b][t][lane];
+#pragma unroll
+        for (int rb = 0; rb < RB; ++rb)
+          acc[rb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wcur[rb][t].v, x.v, acc[rb][b], 0, 0, 0);
+      }
+    if (more) store_acts(buf ^ 1);
+    __syncthreads();
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int t = 0; t < kMidTiles; ++t) wcur[rb][t] = wnext[rb][t];
+  }
+  if (!have_rows) return;
+
+  // lane (j, kg) of accumulator b: token b*16 + j, rows ob*16 + kg*4 + r
+  const int row0 = ob * 16 + kg * 4;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int token = b * 16 + j;
+    if (token >= n || row0 >= m) continue;
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      v[r] = GATED ? silu(acc[0][b][r]) * acc[RB - 1][b][r] : acc[0][b][r];
+      if (bias && row0 + r < m) v[r] += bias[row0 + r];
+    }
+    if (ksplit > 1) {
+      float* o = static_cast<float*>(out) + (static_cast<size_t>(blockIdx.y) * n + token) * ldo + row0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (row0 + r < m) o[r] = v[r];
+      continue;
+    }
+    const size_t idx = static_cast<size_t>(token) * ldo + row0;
+    if (out_f32) {
+      float* o = static_cast<float*>(out) + idx;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+    } else {
+      bf16* o = static_cast<bf16*>(out) + idx;
+      if (row0 + 3 < m && (ldo & 3) == 0) {
+        uint2 packed;
+        packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+        packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+        *reinterpret_cast<uint2*>(o) = packed;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (row0 + r < m) o[r] = from_float<bf16>(v[r]);
+      }
+    }
+  }
+}
+
 // gemm_big_kernel: for many tokens (prompt portions).  A workgroup of 4
 // wavefronts computes 128 weight rows x 128 tokens; each wavefront a 64 x 64
 // quadrant as 4 x 4 MFMA tiles.  Per stage of 64 columns of k, the weights'
@@ -360,7 +511,9 @@ extern "C" int shk_interleave_gate_up(const void* gate_t, const void* up_t, int 
 extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   const int mblocks = (m + 15) / 16, ktiles = (k + 31) / 32;
   if (n > 64 || mblocks >= 512) return 1;
-  int split = 8192 / (mblocks * 4);
+  // up to 16 tokens: workgroups of 4 wavefronts share a block's k-tiles; more tokens:
+  // workgroups of 4 blocks walk k in stages of 4 tiles
+  int split = n <= 16 ? 8192 / (mblocks * 4) : 1024 / ((mblocks + 3) / 4);
   const int most = ktiles / 16;
   if (split > most) split = most;
   if (split > 16) split = 16;
@@ -404,9 +557,37 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }
+  if (n > 16) {
+    // blocks of output rows per workgroup: 8 where that still leaves enough workgroups
+    const int mid_waves = (mb >= 4096) ? 8 : 4;
+    dim3 mgrid((mb + mid_waves - 1) / mid_waves, ksplit);
+#define SHK_MID_W(NB, W)                                                                    \
+  do {                                                                                      \
+    if (gated)                                                                              \
+      gemm_mid_kernel<NB, W, true><<<mgrid, W * kWave, 0, s>>>(                             \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);           \
+    else                                                                                    \
+      gemm_mid_kernel<NB, W, false><<<mgrid, W * kWave, 0, s>>>(                            \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);           \
+  } while (0)
+#define SHK_MID(NB)       \
+  do {                    \
+    if (mid_waves == 8)   \
+      SHK_MID_W(NB, 8);   \
+    else                  \
+      SHK_MID_W(NB, 4);   \
+  } while (0)
+    // always four token blocks: the narrower instantiations measured slower, and the
+    // multiplications for absent tokens cost nothing next to the weight traffic
+    SHK_MID(4);
+#undef SHK_MID
+#undef SHK_MID_W
+    SHK_LAUNCH_CHECK("gemm_bf16");
+    return 0;
+  }
   // wavefronts per workgroup: matrices with few row blocks get more of them
   const int waves = (mb >= 512 || ksplit > 1) ? ((mb >= 512) ? 8 : 4) : 16;
-  const int max_waves = (n > 32 || (gated && n > 16)) ? 8 : 16;  // register budget of the wide variants
+  const int max_waves = 16;
   dim3 sgrid(mb, ksplit);
 #define SHK_SKINNY_W(NB, W)                                                                     \
   do {                                                                                          \
@@ -426,14 +607,7 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     else                                     \
       SHK_SKINNY_W(NB, 16);                  \
   } while (0)
-  if (n <= 16)
-    SHK_SKINNY(1);
-  else if (n <= 32)
-    SHK_SKINNY(2);
-  else if (n <= 48)
-    SHK_SKINNY(3);
-  else
-    SHK_SKINNY(4);
+  SHK_SKINNY(1);
 #undef SHK_SKINNY
 #undef SHK_SKINNY_W
   SHK_LAUNCH_CHECK("gemm_bf16");

@@ -1,9 +1,7 @@
 // Rotary position encoding of queries and keys fused with the write of keys
 // and values into their cache pages.  One thread per element pair (queries and
 // keys) or element (values); a workgroup first tabulates the cosines and sines
-// of its token in LDS.  Angles, sine and cosine are float32 (sincosf with full
-// range reduction: positions reach thousands of radians at the highest
-// frequency).  The projections may arrive as the float32 partial sums of a
+// of its token in LDS.  Angles are float32 products as in the reference.  The projections may arrive as the float32 partial sums of a
 // product that was split along k; they are added here, in order, with the bias.
 #include "api.h"
 #include "common.h"
@@ -30,8 +28,15 @@ __global__ void __launch_bounds__(kRopeThreads)
   const int half = rot_dim / 2;
   const int width = (heads + 2 * kv_heads) * head_dim;
   for (int i = threadIdx.x; i < half; i += kRopeThreads) {
+    // The angle is the float32 product, as the reference forms it; it reaches
+    // thousands of radians, so it is brought into [-pi, pi] in float64 (exact
+    // to 1e-13) before the float32 sine and cosine.
+    const float angle = static_cast<float>(pos) * inv_freq[i];
+    const double a = static_cast<double>(angle);
+    const double turns = rint(a * 0.15915494309189535);
+    const float reduced = static_cast<float>(fma(turns, -6.283185307179586, a));
     float s, c;
-    sincosf(static_cast<float>(pos) * inv_freq[i], &s, &c);
+    sincosf(reduced, &s, &c);
     cs[i] = c;
     sn[i] = s;
   }

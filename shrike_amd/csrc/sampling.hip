@@ -56,6 +56,36 @@ __global__ void __launch_bounds__(kSampleThreads)
   if (threadIdx.x == 0) out[blockIdx.x] = best.i;
 }
 
+// Two stages for wide rows: every chunk of kArgmaxChunk values gets a workgroup
+// that leaves its best (value, index); a second kernel picks among the chunks,
+// lowest index first among equals.
+constexpr int kArgmaxChunk = 4096;
+constexpr int kArgmaxThreads = 256;
+
+__global__ void __launch_bounds__(kArgmaxThreads)
+    argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ best_value,
+                         int32_t* __restrict__ best_index, int vocab, int ld, int chunks) {
+  __shared__ MaxIdx scratch[16];
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const int begin = chunk * kArgmaxChunk;
+  const int count = vocab - begin < kArgmaxChunk ? vocab - begin : kArgmaxChunk;
+  MaxIdx best = block_argmax(logits + static_cast<size_t>(row) * ld + begin, count, scratch);
+  if (threadIdx.x == 0) {
+    best_value[row * chunks + chunk] = best.v;
+    best_index[row * chunks + chunk] = begin + best.i;
+  }
+}
+
+__global__ void __launch_bounds__(kArgmaxThreads)
+    argmax_pick_kernel(const float* __restrict__ best_value, const int32_t* __restrict__ best_index,
+                       int32_t* __restrict__ out, int chunks) {
+  __shared__ MaxIdx scratch[16];
+  const int row = blockIdx.x;
+  // chunks are in index order, so the first maximum among them has the lowest index
+  const MaxIdx best = block_argmax(best_value + static_cast<size_t>(row) * chunks, chunks, scratch);
+  if (threadIdx.x == 0) out[row] = best_index[row * chunks + best.i];
+}
+
 // Exclusive prefix sums over the threads of the workgroup (thread order), and the total.
 __device__ void block_exclusive_scan(float v, float* buf, float* before, float* total) {
   __syncthreads();
@@ -187,14 +217,32 @@ __global__ void __launch_bounds__(kSampleThreads)
 
 using namespace shk;
 
+extern "C" int shk_argmax_scratch_floats(int rows, int vocab) {
+  const int chunks = (vocab + kArgmaxChunk - 1) / kArgmaxChunk;
+  return chunks > 1 ? 2 * rows * chunks : 0;
+}
+
 extern "C" int shk_argmax(const float* logits, int32_t* out, int rows, int vocab, int ld,
-                          void* stream) {
+                          float* scratch, void* stream) {
   SHK_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "argmax: bad sizes rows=%d vocab=%d ld=%d",
               rows, vocab, ld);
   if (rows == 0) return 0;
   SHK_REQUIRE(logits && out, "argmax: null pointer");
-  argmax_kernel<<<rows, kSampleThreads, 0, static_cast<hipStream_t>(stream)>>>(logits, out, vocab,
-                                                                               ld);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int chunks = (vocab + kArgmaxChunk - 1) / kArgmaxChunk;
+  if (chunks == 1) {
+    argmax_kernel<<<rows, kSampleThreads, 0, s>>>(logits, out, vocab, ld);
+    SHK_LAUNCH_CHECK("argmax");
+    return 0;
+  }
+  SHK_REQUIRE(scratch, "argmax: rows of %d values need the scratch buffer", vocab);
+  SHK_REQUIRE(rows <= 65535, "argmax: at most 65535 rows a call, got %d", rows);
+  float* best_value = scratch;
+  int32_t* best_index = reinterpret_cast<int32_t*>(scratch + static_cast<size_t>(rows) * chunks);
+  argmax_chunks_kernel<<<dim3(chunks, rows), kArgmaxThreads, 0, s>>>(logits, best_value, best_index,
+                                                                     vocab, ld, chunks);
+  SHK_LAUNCH_CHECK("argmax");
+  argmax_pick_kernel<<<rows, kArgmaxThreads, 0, s>>>(best_value, best_index, out, chunks);
   SHK_LAUNCH_CHECK("argmax");
   return 0;
 }

@@ -121,9 +121,11 @@ class ModelRunner:
                     raise StepError(
                         f"block table has {len(table)} pages but the step reaches page {last_page}"
                     )
+                # the pages this step writes, and the oldest page it reads
                 w = g.spec.window
                 first = 0 if w is None else max(0, e.start - w + 1) // ps
-                if any(p < 0 or p >= self.cache.num_pages for p in table[first : last_page + 1]):
+                touched = table[e.start // ps : last_page + 1]
+                if min(touched) < 0 or max(touched) >= self.cache.num_pages or table[first] < 0:
                     raise StepError("block table names a page outside the pool")
 
     def _meta(self, entries: list[StepEntry], order: list[int], pad_to: int = 0,

@@ -317,12 +317,24 @@ def attention_prefill(q, out, num_tiles, heads, kv_heads, head_dim, cu_q, ctx_le
     )
 
 
+_ARGMAX_SCRATCH: dict = {}
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     """out[r] = lowest index of the maximum of logits[r]; logits float32 [rows, vocab]."""
     _rows(logits, "argmax logits")
     rows, vocab = logits.shape
+    need = load().shk_argmax_scratch_floats(rows, vocab)
+    scratch = None
+    if need:
+        key = (logits.device.type, logits.device.index)
+        scratch = _ARGMAX_SCRATCH.get(key)
+        if scratch is None or scratch.numel() < need:
+            scratch = torch.empty(max(need, 1 << 16), dtype=torch.float32, device=logits.device)
+            _ARGMAX_SCRATCH[key] = scratch
     check(load().shk_argmax(_dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32),
-                            rows, vocab, logits.stride(0), _stream()))
+                            rows, vocab, logits.stride(0),
+                            None if scratch is None else scratch.data_ptr(), _stream()))
 
 
 def sample(logits, out, temperature, top_p, uniforms, scratch) -> None:
