@@ -31,6 +31,29 @@ union AFrag {
   uint16_t h[8];
 };
 
+// Maximum and sum over the 16 lanes that hold one row of a score tile (lanes
+// 16*g .. 16*g+15, a DPP "row"): four data-parallel-primitive moves on the vector
+// unit instead of four round trips through the LDS crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float row16_max(float v) {
+  v = fmaxf(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]: lane ^ 1
+  v = fmaxf(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]: lane ^ 2
+  v = fmaxf(v, dpp_move<0x141>(v));  // row_half_mirror: the other quad of each 8 lanes
+  v = fmaxf(v, dpp_move<0x140>(v));  // row_mirror: the other half of the 16 lanes
+  return v;
+}
+__device__ __forceinline__ float row16_sum(float v) {
+  v += dpp_move<0xB1>(v);
+  v += dpp_move<0x4E>(v);
+  v += dpp_move<0x141>(v);
+  v += dpp_move<0x140>(v);
+  return v;
+}
+
 constexpr int kPStride = 40;  // bf16 elements per row of the P tile in LDS (32 + padding)
 
 // A window of 64 entries of a sequence's block table held across the lanes of
@@ -162,17 +185,13 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
         const bool keep = key <= row_pos[r] && key >= row_lo[r];
         sc[tt] = keep ? s[tt][r] * ta.scale : -INFINITY;
       }
-      float mx = fmaxf(sc[0], sc[1]);
-#pragma unroll
-      for (int off = 1; off < 16; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, kWave));
+      const float mx = row16_max(fmaxf(sc[0], sc[1]));
       const float m_new = fmaxf(m[r], mx);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __expf(m[r] - m_safe);
       p[0][r] = __expf(sc[0] - m_safe);
       p[1][r] = __expf(sc[1] - m_safe);
-      float sum = p[0][r] + p[1][r];
-#pragma unroll
-      for (int off = 1; off < 16; off <<= 1) sum += __shfl_xor(sum, off, kWave);
+      const float sum = row16_sum(p[0][r] + p[1][r]);
       l[r] = l[r] * alpha + sum;
       m[r] = m_new;
 #pragma unroll
@@ -319,7 +338,7 @@ __global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* 
 // its first query inside the sequence's portion.
 
 template <int D>
-__global__ void __launch_bounds__(kWave)
+__global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
     attention_prefill_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                              int heads, int kv_heads, const int32_t* __restrict__ cu_q,
                              const int32_t* __restrict__ ctx_lens,
@@ -329,7 +348,8 @@ __global__ void __launch_bounds__(kWave)
                              const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
                              int page_size, int window, float scale) {
   __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * kPStride];
-  const int tile = blockIdx.x, head = blockIdx.y;
+  // tiles are listed in token order; the last ones read the most keys, so they start first
+  const int tile = gridDim.x - 1 - blockIdx.x, head = blockIdx.y;
   const int lane = threadIdx.x, j = lane % 16, kg = lane / 16;
   const int seq = tile_seq[tile], q0 = tile_q0[tile];
   const int tok0 = cu_q[seq], q_len = cu_q[seq + 1] - tok0;
@@ -379,6 +399,215 @@ __global__ void __launch_bounds__(kWave)
   }
 }
 
+// ------------------------------------------------- prefill, keys shared in LDS
+// A workgroup of 4 wavefronts serves every query head of one key/value head for
+// a run of 16-query tiles of one sequence: the chunk of 32 keys is fetched once,
+// staged in LDS in operand layout and read by all of them, instead of once per
+// (head, tile).  A wavefront owns two "units" (query head, query tile); unit
+// u < tiles * group is tile u / group, head u % group of the key/value head.
+// grid (workgroup tiles, kv_heads); wg_seq / wg_q0 as tile_seq / tile_q0 above,
+// in steps of 16 * tiles queries.
+
+constexpr int kUnitsPerWave = 2;
+constexpr int kSharedWaves = 4;
+
+template <int D>
+__global__ void __launch_bounds__(kSharedWaves* kWave) __attribute__((amdgpu_waves_per_eu(2)))
+    attention_prefill_shared_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+                                    int heads, int kv_heads, int tiles,
+                                    const int32_t* __restrict__ cu_q,
+                                    const int32_t* __restrict__ ctx_lens,
+                                    const int32_t* __restrict__ wg_seq,
+                                    const int32_t* __restrict__ wg_q0,
+                                    const int32_t* __restrict__ tables, int table_stride,
+                                    const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
+                                    int page_size, int window, float scale) {
+  constexpr int kKFrags = 2 * (D / 32), kVFrags = D / 16, kFrags = kKFrags + kVFrags;
+  constexpr int kPerThread = kFrags / kSharedWaves;  // fragments each wavefront stages
+  __shared__ uint4 kv[2][kFrags][kWave];
+  __shared__ __attribute__((aligned(16))) uint16_t p_all[kSharedWaves][16 * kPStride];
+
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int j = lane % 16, kg = lane / 16;
+  // workgroups are listed in token order; the last ones read the most keys, so they start first
+  const int wg = gridDim.x - 1 - blockIdx.x;
+  const int seq = wg_seq[wg], q0 = wg_q0[wg], kvh = blockIdx.y;
+  const int group = heads / kv_heads;
+  const int tok0 = cu_q[seq], q_len = cu_q[seq + 1] - tok0;
+  const int start = ctx_lens[seq] - q_len;  // position of the portion's first token
+  const int q_end = (q0 + 16 * tiles < q_len) ? q0 + 16 * tiles : q_len;
+  const int ps = page_size;
+  const size_t head_elems = static_cast<size_t>(ps) * D;
+  const int32_t* table = tables + static_cast<size_t>(seq) * table_stride;
+  uint16_t* p_lds = p_all[wave];
+
+  // bounds over the whole workgroup: what has to be staged
+  const int pos_min = start + q0, pos_max = start + q_end - 1;
+  const int lo_min = (window > 0 && pos_min - window + 1 > 0) ? pos_min - window + 1 : 0;
+  const int key_begin = lo_min & ~31;
+
+  // this wavefront's units
+  AFrag qf[kUnitsPerWave][D / 32];
+  int row_pos[kUnitsPerWave][4], row_lo[kUnitsPerWave][4];
+  float m[kUnitsPerWave][4], l[kUnitsPerWave][4];
+  f32x4 o[kUnitsPerWave][D / 16];
+  int unit_head[kUnitsPerWave], unit_q0[kUnitsPerWave], unit_rows[kUnitsPerWave];
+#pragma unroll
+  for (int u = 0; u < kUnitsPerWave; ++u) {
+    const int unit = wave * kUnitsPerWave + u;
+    const bool valid = unit < tiles * group && q0 + (unit / group) * 16 < q_len;
+    unit_head[u] = kvh * group + unit % group;
+    unit_q0[u] = q0 + (unit / group) * 16;
+    unit_rows[u] = !valid ? 0 : (q_len - unit_q0[u] < 16 ? q_len - unit_q0[u] : 16);
+    const bf16* qrow = q + static_cast<size_t>(tok0 + unit_q0[u] + j) * q_stride +
+                       static_cast<size_t>(unit_head[u]) * D + kg * 8;
+#pragma unroll
+    for (int ds = 0; ds < D / 32; ++ds) {
+      qf[u][ds].u = make_uint4(0, 0, 0, 0);
+      if (j < unit_rows[u]) qf[u][ds].u = *reinterpret_cast<const uint4*>(qrow + ds * 32);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int qi = kg * 4 + r;
+      row_pos[u][r] = (qi < unit_rows[u]) ? start + unit_q0[u] + qi : -1;
+      row_lo[u][r] = (window > 0 && row_pos[u][r] - window + 1 > 0) ? row_pos[u][r] - window + 1 : 0;
+      m[u][r] = -INFINITY;
+      l[u][r] = 0.f;
+    }
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) o[u][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // Staging: wavefront w fetches fragments w, w + 4, ...  Fragment f < kKFrags is
+  // K tile f / (D/32), head_dim slice f % (D/32); the others are V blocks of 16 elements.
+  uint4 regs[kPerThread];
+  auto fetch = [&](int kb) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) {
+      const int f = wave + kSharedWaves * i;
+      regs[i] = make_uint4(0, 0, 0, 0);
+      if (f < kKFrags) {
+        const int tt = f / (D / 32), ds = f % (D / 32);
+        const int key0 = kb + tt * 16;
+        if (key0 <= pos_max && key0 + 15 >= lo_min) {
+          const int page = table[key0 / ps];
+          regs[i] = *reinterpret_cast<const uint4*>(
+              k_pool + (static_cast<size_t>(page) * kv_heads + kvh) * head_elems +
+              static_cast<size_t>(key0 % ps + j) * D + ds * 32 + kg * 8);
+        }
+      } else {
+        const int db = f - kKFrags;
+        const int g0 = kb + kg * 8;
+        if (g0 <= pos_max && g0 + 7 >= lo_min) {
+          const int page = table[g0 / ps];
+          uint4 v = *reinterpret_cast<const uint4*>(
+              v_pool + (static_cast<size_t>(page) * kv_heads + kvh) * head_elems +
+              static_cast<size_t>(db * 16 + j) * ps + g0 % ps);
+          if (g0 < lo_min || g0 + 7 > pos_max) {
+            // keys outside [lo_min, pos_max] carry weight 0 but may hold anything
+            uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const bool a = g0 + 2 * e >= lo_min && g0 + 2 * e <= pos_max;
+              const bool b = g0 + 2 * e + 1 >= lo_min && g0 + 2 * e + 1 <= pos_max;
+              w[e] &= (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
+            }
+            v = make_uint4(w[0], w[1], w[2], w[3]);
+          }
+          regs[i] = v;
+        }
+      }
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kPerThread; ++i) kv[buf][wave + kSharedWaves * i][lane] = regs[i];
+  };
+
+  fetch(key_begin);
+  stash(0);
+  __syncthreads();
+  int buf = 0;
+  for (int kb = key_begin; kb <= pos_max; kb += 32) {
+    const bool more = kb + 32 <= pos_max;
+    if (more) fetch(kb + 32);
+#pragma unroll
+    for (int u = 0; u < kUnitsPerWave; ++u) {
+      // ---- S = Q K^T
+      f32x4 s[2];
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt) {
+        s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ds = 0; ds < D / 32; ++ds) {
+          AFrag kf;
+          kf.u = kv[buf][tt * (D / 32) + ds][lane];
+          s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u][ds].v, kf.v, s[tt], 0, 0, 0);
+        }
+      }
+      // ---- mask, running maximum and sum
+      float p[2][4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float sc[2];
+#pragma unroll
+        for (int tt = 0; tt < 2; ++tt) {
+          const int key = kb + tt * 16 + j;
+          const bool keep = key <= row_pos[u][r] && key >= row_lo[u][r];
+          sc[tt] = keep ? s[tt][r] * scale : -INFINITY;
+        }
+        const float mx = row16_max(fmaxf(sc[0], sc[1]));
+        const float m_new = fmaxf(m[u][r], mx);
+        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __expf(m[u][r] - m_safe);
+        p[0][r] = __expf(sc[0] - m_safe);
+        p[1][r] = __expf(sc[1] - m_safe);
+        const float sum = row16_sum(p[0][r] + p[1][r]);
+        l[u][r] = l[u][r] * alpha + sum;
+        m[u][r] = m_new;
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db) o[u][db][r] *= alpha;
+      }
+      // ---- P through this wavefront's LDS patch into A-operand layout.  Only this
+      // wavefront touches the patch; the fences order its own writes and reads.
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          p_lds[(kg * 4 + r) * kPStride + tt * 16 + j] = bf16_bits(p[tt][r]);
+      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      AFrag pf;
+      pf.u = *reinterpret_cast<const uint4*>(p_lds + j * kPStride + kg * 8);
+      // ---- O += P V
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db) {
+        AFrag vf;
+        vf.u = kv[buf][kKFrags + db][lane];
+        o[u][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, o[u][db], 0, 0, 0);
+      }
+    }
+    if (more) stash(buf ^ 1);
+    __syncthreads();
+    buf ^= 1;
+  }
+
+#pragma unroll
+  for (int u = 0; u < kUnitsPerWave; ++u)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int qi = kg * 4 + r;
+      if (qi >= unit_rows[u]) continue;
+      bf16* dst = out + static_cast<size_t>(tok0 + unit_q0[u] + qi) * heads * D +
+                  static_cast<size_t>(unit_head[u]) * D;
+      const float inv = 1.f / l[u][r];
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db) dst[db * 16 + j] = from_float<bf16>(o[u][db][r] * inv);
+    }
+}
+
 template <int D>
 static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, int heads,
                           int kv_heads, const int32_t* positions, const int32_t* tables,
@@ -399,6 +628,18 @@ static void launch_prefill(dim3 grid, hipStream_t s, const bf16* q, int q_stride
                                                      ctx_lens, tile_seq, tile_q0, tables,
                                                      table_stride, k_pool, v_pool, page_size,
                                                      window, scale);
+}
+
+template <int D>
+static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q_stride, bf16* out,
+                                  int heads, int kv_heads, int tiles, const int32_t* cu_q,
+                                  const int32_t* ctx_lens, const int32_t* wg_seq,
+                                  const int32_t* wg_q0, const int32_t* tables, int table_stride,
+                                  const bf16* k_pool, const bf16* v_pool, int page_size, int window,
+                                  float scale) {
+  attention_prefill_shared_kernel<D><<<grid, kSharedWaves * kWave, 0, s>>>(
+      q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables, table_stride,
+      k_pool, v_pool, page_size, window, scale);
 }
 
 }  // namespace shk
@@ -464,6 +705,53 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
   attention_merge_kernel<<<num_seqs * heads, head_dim <= 64 ? 64 : 128, 0, s>>>(
       partial, static_cast<bf16*>(out), head_dim, nsplit);
   SHK_LAUNCH_CHECK("attention_merge");
+  return 0;
+}
+
+// Query tiles of 16 that one workgroup of the shared-key prefill kernel serves for
+// a given number of query heads per key/value head; 0: the shape is not served.
+extern "C" int shk_attention_prefill_shared_tiles(int heads, int kv_heads, int head_dim) {
+  const int group = heads / kv_heads;
+  if (group < 1 || group > kUnitsPerWave * kSharedWaves || head_dim > 128) return 0;
+  return (kUnitsPerWave * kSharedWaves) / group;
+}
+
+extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out,
+                                                 int num_wgs, int heads, int kv_heads,
+                                                 int head_dim, const int32_t* cu_q,
+                                                 const int32_t* ctx_lens, const int32_t* wg_seq,
+                                                 const int32_t* wg_q0, const int32_t* tables,
+                                                 int table_stride, const void* k_pool,
+                                                 const void* v_pool, int page_size, int window,
+                                                 float scale, void* stream) {
+  if (check_mfma_shapes("attention_prefill_shared", heads, kv_heads, head_dim, page_size, q_stride))
+    return 1;
+  const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim);
+  SHK_REQUIRE(tiles > 0, "attention_prefill_shared: %d query heads per key/value head or head_dim %d "
+              "is not served", heads / kv_heads, head_dim);
+  SHK_REQUIRE(num_wgs >= 0 && kv_heads <= 65535, "attention_prefill_shared: bad sizes");
+  if (num_wgs == 0) return 0;
+  SHK_REQUIRE(q && out && cu_q && ctx_lens && wg_seq && wg_q0 && tables && k_pool && v_pool &&
+                  table_stride > 0,
+              "attention_prefill_shared: null pointer");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0,
+              "attention_prefill_shared: q is not 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  dim3 grid(num_wgs, kv_heads);
+#define CALL(D)                                                                                \
+  launch_prefill_shared<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
+                           heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,      \
+                           table_stride, static_cast<const bf16*>(k_pool),                     \
+                           static_cast<const bf16*>(v_pool), page_size, window, scale)
+  switch (head_dim) {
+    case 32: CALL(32); break;
+    case 64: CALL(64); break;
+    case 96: CALL(96); break;
+    case 128: CALL(128); break;
+    default: break;
+  }
+#undef CALL
+  SHK_LAUNCH_CHECK("attention_prefill_shared");
   return 0;
 }
 

@@ -327,64 +327,65 @@ __global__ void __launch_bounds__(WAVES* kWave)
 }
 
 // gemm_big_kernel: for many tokens (prompt portions).  A workgroup of 4
-// wavefronts computes 128 weight rows x 128 tokens; each wavefront a 64 x 64
-// quadrant as 4 x 4 MFMA tiles.  Per stage of 64 columns of k, the weights'
-// tiles (already in operand layout) and the activations (re-laid on the way)
+// wavefronts computes a tile of weight rows x tokens, each wavefront a
+// quadrant of it as WM x WN MFMA tiles.  Per stage of k, the weights' tiles (already in operand layout) and the activations (re-laid on the way)
 // are staged in LDS "fragment-major": the 16 bytes of lane l of a fragment sit
 // at l * 16, so every LDS access is a conflict-free 128-bit access.  Stages are
 // double-buffered: the loads of stage t+1 are in flight while stage t is
 // multiplied.
 
-constexpr int kBigM = 128;   // weight rows per workgroup
-constexpr int kBigN = 128;   // tokens per workgroup
-constexpr int kBigK = 64;    // k per stage (two MFMA steps)
-constexpr int kBigFrags = (kBigM / 16) * (kBigK / 32);  // fragments per operand per stage: 16
-
-template <bool GATED>
+// WM x WN: MFMA tiles (16 x 16) per wavefront; the workgroup's 2 x 2 wavefronts
+// cover 32*WM weight rows x 32*WN tokens.  KS: MFMA steps (32 of k) per stage.
+template <int WM, int WN, int KS, bool GATED>
 __global__ void __launch_bounds__(256)
     gemm_big_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                     const uint4* __restrict__ wt, int ktiles, int m,
                     const float* __restrict__ bias, void* __restrict__ out, int ldo, int out_f32,
                     int accumulate, int vec) {
-  // [buffer][operand: 0 weights, 1 activations][fragment][lane]
-  __shared__ uint4 stage[2][2][kBigFrags][kWave];
+  constexpr int kWFrags = 2 * WM * KS, kAFrags = 2 * WN * KS;  // fragments per stage
+  // [buffer][fragment][lane]: weights first, then activations
+  __shared__ uint4 stage[2][kWFrags + kAFrags][kWave];
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wm = wave / 2, wn = wave % 2;  // quadrant of the wavefront
-  const int mb0 = blockIdx.x * (kBigM / 16);   // first block of 16 weight rows
-  const int tok0 = blockIdx.y * kBigN;
+  const int mb0 = blockIdx.x * (2 * WM);   // first block of 16 weight rows
+  const int tok0 = blockIdx.y * (32 * WN);
   // blocks of 16 weight rows; a gated weight has two per 16 output rows
   const int mblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
-  const int nstages = (ktiles + 1) / 2;
+  const int nstages = (ktiles + KS - 1) / KS;
 
-  f32x4 acc[4][4];
+  f32x4 acc[WM][WN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int jn = 0; jn < 4; ++jn) acc[i][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int jn = 0; jn < WN; ++jn) acc[i][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // Each thread moves 4 fragments-lanes per operand per stage: fragment f = tid/64 + 4*i
-  // (f = rb * 2 + ks: block of 16 rows rb, MFMA step ks), lane = tid % 64.
-  uint4 wreg[4], areg[4];
+  // Fragment f of an operand is (block of 16 rows f / KS, MFMA step f % KS); wavefront w
+  // moves fragments w, w + 4, ...
+  constexpr int kWPer = (kWFrags + 3) / 4, kAPer = (kAFrags + 3) / 4;
+  uint4 wreg[kWPer], areg[kAPer];
   auto load_stage = [&](int st) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int f = wave + 4 * i, rb = f / 2, ks = f % 2;
-      const int kt = st * 2 + ks;
-      const int mb = mb0 + rb;
+    for (int i = 0; i < kWPer; ++i) {
+      const int f = wave + 4 * i, rb = f / KS, kt = st * KS + f % KS;
       wreg[i] = make_uint4(0, 0, 0, 0);
-      if (mb < mblocks && kt < ktiles)
-        wreg[i] = wt[(static_cast<size_t>(mb) * ktiles + kt) * kWave + lane];
-      const int token = tok0 + rb * 16 + lane % 16;
-      areg[i] = load_act(a, lda, n, k, token, kt * 32 + (lane / 16) * 8, vec).u;
+      if (f < kWFrags && mb0 + rb < mblocks && kt < ktiles)
+        wreg[i] = wt[(static_cast<size_t>(mb0 + rb) * ktiles + kt) * kWave + lane];
+    }
+#pragma unroll
+    for (int i = 0; i < kAPer; ++i) {
+      const int f = wave + 4 * i, rb = f / KS, kt = st * KS + f % KS;
+      areg[i] = make_uint4(0, 0, 0, 0);
+      if (f < kAFrags)
+        areg[i] = load_act(a, lda, n, k, tok0 + rb * 16 + lane % 16, kt * 32 + (lane / 16) * 8, vec).u;
     }
   };
   auto store_stage = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int f = wave + 4 * i;
-      stage[buf][0][f][lane] = wreg[i];
-      stage[buf][1][f][lane] = areg[i];
-    }
+    for (int i = 0; i < kWPer; ++i)
+      if (wave + 4 * i < kWFrags) stage[buf][wave + 4 * i][lane] = wreg[i];
+#pragma unroll
+    for (int i = 0; i < kAPer; ++i)
+      if (wave + 4 * i < kAFrags) stage[buf][kWFrags + wave + 4 * i][lane] = areg[i];
   };
 
   load_stage(0);
@@ -394,32 +395,34 @@ __global__ void __launch_bounds__(256)
     const int buf = st & 1;
     if (st + 1 < nstages) load_stage(st + 1);
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      Frag wf[4], af[4];
+    for (int ks = 0; ks < KS; ++ks) {
+      Frag af[WN];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) wf[i].u = stage[buf][0][(wm * 4 + i) * 2 + ks][lane];
+      for (int jn = 0; jn < WN; ++jn) af[jn].u = stage[buf][kWFrags + (wn * WN + jn) * KS + ks][lane];
 #pragma unroll
-      for (int jn = 0; jn < 4; ++jn) af[jn].u = stage[buf][1][(wn * 4 + jn) * 2 + ks][lane];
+      for (int i = 0; i < WM; ++i) {
+        Frag wf;
+        wf.u = stage[buf][(wm * WM + i) * KS + ks][lane];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int jn = 0; jn < 4; ++jn)
-          acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i].v, af[jn].v, acc[i][jn], 0, 0, 0);
+        for (int jn = 0; jn < WN; ++jn)
+          acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, af[jn].v, acc[i][jn], 0, 0, 0);
+      }
     }
     if (st + 1 < nstages) store_stage(buf ^ 1);
     __syncthreads();
   }
 
-  // lane (j, kg) of tile (i, jn): token tok0 + (wn*4 + jn)*16 + j, rows (mb0 + wm*4 + i)*16 + kg*4 + r
+  // lane (j, kg) of tile (i, jn): token tok0 + (wn*WN + jn)*16 + j,
+  // rows (mb0 + wm*WM + i)*16 + kg*4 + r
   const int j = lane % 16, kg = lane / 16;
 #pragma unroll
-  for (int jn = 0; jn < 4; ++jn) {
-    const int token = tok0 + (wn * 4 + jn) * 16 + j;
+  for (int jn = 0; jn < WN; ++jn) {
+    const int token = tok0 + (wn * WN + jn) * 16 + j;
     if (token >= n) continue;
 #pragma unroll
-    for (int i = 0; i < 4; i += (GATED ? 2 : 1)) {
+    for (int i = 0; i < WM; i += (GATED ? 2 : 1)) {
       // gated: weight blocks come in (gate, up) pairs that make one block of output rows
-      const int row0 = (GATED ? (mb0 + wm * 4 + i) / 2 : mb0 + wm * 4 + i) * 16 + kg * 4;
+      const int row0 = (GATED ? (mb0 + wm * WM + i) / 2 : mb0 + wm * WM + i) * 16 + kg * 4;
       if (row0 >= m) continue;
       float v[4];
 #pragma unroll
@@ -544,22 +547,32 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   const int of = out_dtype == kF32;
   if (n > 64) {
     SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
-    dim3 grid((m + kBigM - 1) / kBigM, (n + kBigN - 1) / kBigN);
-    SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);
-    if (gated) {
-      grid.x = (2 * mb * 16 + kBigM - 1) / kBigM;
-      gemm_big_kernel<true><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,
-                                                 accumulate, vec);
-    } else {
-      gemm_big_kernel<false><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,
-                                                  accumulate, vec);
-    }
+    const int wblocks = (gated ? 2 : 1) * mb;  // blocks of 16 weight rows
+#define SHK_BIG(WM, WN, KS)                                                                  \
+  do {                                                                                       \
+    dim3 grid((wblocks + 2 * WM - 1) / (2 * WM), (n + 32 * WN - 1) / (32 * WN));            \
+    SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);                        \
+    if (gated)                                                                               \
+      gemm_big_kernel<WM, WN, KS, true><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, \
+                                                             out, ldo, of, accumulate, vec); \
+    else                                                                                     \
+      gemm_big_kernel<WM, WN, KS, false><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, \
+                                                              out, ldo, of, accumulate, vec); \
+  } while (0)
+    // 128 x 128 per workgroup, 64 of k per stage.  (Tiles of 256 rows measured slower:
+    // their accumulators no longer fit the register file.)
+    SHK_BIG(4, 4, 2);
+#undef SHK_BIG
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }
   if (n > 16) {
     // blocks of output rows per workgroup: 8 where that still leaves enough workgroups
+#ifdef SHK_MID_WAVES
+    const int mid_waves = (mb >= 4096) ? 8 : SHK_MID_WAVES;
+#else
     const int mid_waves = (mb >= 4096) ? 8 : 4;
+#endif
     dim3 mgrid((mb + mid_waves - 1) / mid_waves, ksplit);
 #define SHK_MID_W(NB, W)                                                                    \
   do {                                                                                      \
@@ -570,12 +583,14 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
       gemm_mid_kernel<NB, W, false><<<mgrid, W * kWave, 0, s>>>(                            \
           ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);           \
   } while (0)
-#define SHK_MID(NB)       \
-  do {                    \
-    if (mid_waves == 8)   \
-      SHK_MID_W(NB, 8);   \
-    else                  \
-      SHK_MID_W(NB, 4);   \
+#define SHK_MID(NB)          \
+  do {                       \
+    if (mid_waves == 8)      \
+      SHK_MID_W(NB, 8);      \
+    else if (mid_waves == 2) \
+      SHK_MID_W(NB, 2);      \
+    else                     \
+      SHK_MID_W(NB, 4);      \
   } while (0)
     // always four token blocks: the narrower instantiations measured slower, and the
     // multiplications for absent tokens cost nothing next to the weight traffic

@@ -72,5 +72,22 @@ class StepContext:
     tile_q0: torch.Tensor | None = None
     num_prefill_tiles: int = 0
 
+    _wg_cache: dict = field(default_factory=dict)
+
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)
+
+    def prefill_workgroups(self, tiles: int):
+        """Prompt portions cut into runs of `tiles` 16-query tiles: (sequence of
+        each run, its first query, number of runs), on the device."""
+        hit = self._wg_cache.get(tiles)
+        if hit is None:
+            seqs, q0s = [], []
+            for s in range(self.num_decode, self.num_seqs):
+                for q0 in range(0, self.q_lens[s], 16 * tiles):
+                    seqs.append(s)
+                    q0s.append(q0)
+            both = torch.tensor([seqs, q0s], dtype=torch.int32).to(self.device)
+            hit = (both[0], both[1], len(seqs))
+            self._wg_cache[tiles] = hit
+        return hit

@@ -317,6 +317,34 @@ def attention_prefill(q, out, num_tiles, heads, kv_heads, head_dim, cu_q, ctx_le
     )
 
 
+def attention_prefill_shared_tiles(heads, kv_heads, head_dim) -> int:
+    """16-query tiles per workgroup of attention_prefill_shared; 0 if the shape is not served."""
+    return int(load().shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim))
+
+
+def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, ctx_lens, wg_seq, wg_q0,
+                             tables, k_pool, v_pool, page_size, window, scale) -> None:
+    """bfloat16 MFMA attention for prompt portions; one workgroup per (run of query
+    tiles, key/value head) shares each chunk of keys among its query heads."""
+    _rows(q, "attention_prefill_shared q")
+    if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
+        raise KernelError("attention_prefill_shared: bfloat16 only")
+    if out.shape != (q.shape[0], heads * head_dim) or not out.is_contiguous():
+        raise KernelError("attention_prefill_shared: out must be contiguous [n, heads*head_dim]")
+    if wg_seq.shape[0] < num_wgs or wg_q0.shape[0] < num_wgs:
+        raise KernelError("attention_prefill_shared: workgroup arrays are shorter than num_wgs")
+    _check_pools("attention_prefill_shared", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
+    check(
+        load().shk_attention_prefill_shared_bf16(
+            _dev(q, "q"), q.stride(0), _dev(out, "out"), num_wgs, heads, kv_heads, head_dim,
+            _dev(cu_q, "cu_q", torch.int32), _dev(ctx_lens, "ctx_lens", torch.int32),
+            _dev(wg_seq, "wg_seq", torch.int32), _dev(wg_q0, "wg_q0", torch.int32),
+            _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
+            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), _stream(),
+        )
+    )
+
+
 _ARGMAX_SCRATCH: dict = {}
 
 

@@ -587,3 +587,46 @@ def test_rope_kv_store_adds_up_a_split_product(ops):
         page = int(tables[t, p // page_size])
         close(k_pool[page, :, p % page_size], k[t], dtype)
         close(v_pool[page, :, :, p % page_size], v[t], dtype)
+
+
+@pytest.mark.parametrize(
+    "heads, kv_heads, head_dim, page_size, window",
+    [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 128, 16, None),
+     (16, 2, 64, 16, 100), (3, 1, 128, 48, None)],
+)
+def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window):
+    """The prefill kernel that shares each chunk of keys among the query heads of a
+    key/value head: 1 to 8 heads per group, portions of 2 to 200 tokens."""
+    torch.manual_seed(20)
+    dtype = torch.bfloat16
+    tiles = ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim)
+    assert tiles == 8 // (heads // kv_heads)
+    seq_lens = [2, 200, 16, 17, 90, 33, 130]
+    starts = [0, 60, 5, 100, 0, 31, 7]
+    ctx = [s + l for s, l in zip(starts, seq_lens)]
+    n = sum(seq_lens)
+    num_pages = sum(-(-c // page_size) for c in ctx) + 5
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, num_pages, kv_heads, head_dim, dtype, seed=5)
+    fill_pools(tables, k_pool, v_pool, ctx, page_size)
+    q = torch.randn(n, heads, head_dim).to(dtype)
+    cu = [0]
+    for l in seq_lens:
+        cu.append(cu[-1] + l)
+    wg_seq, wg_q0 = [], []
+    for s, l in enumerate(seq_lens):
+        for q0 in range(0, l, 16 * tiles):
+            wg_seq.append(s)
+            wg_q0.append(q0)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
+    scale = head_dim**-0.5
+    ops.attention_prefill_shared(dev(q).view(n, -1), out, len(wg_seq), heads, kv_heads, head_dim, i32(cu), i32(ctx),
+                                 i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, window, scale)
+    want = reference_attention(q.double(), k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale)
+    assert not torch.isnan(out.float()).any()
+    close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
+
+
+def test_attention_prefill_shared_refuses_wide_groups(ops):
+    assert ops.attention_prefill_shared_tiles(32, 2, 64) == 0  # 16 heads per group: the per-tile kernel serves it
+    assert ops.attention_prefill_shared_tiles(8, 2, 256) == 0
