@@ -75,6 +75,13 @@ class _DecodeGraph:
         self.meta_dev = None
         self.logits = None
         self.ctx = None
+        # host copy of the metadata, updated in place from step to step
+        self.pinned = None
+        self.host = None  # numpy view of `pinned`
+        self.copied = None  # event: the last copy out of `pinned` is done
+        self.offsets = None  # field -> offset in the buffer; tables -> list of offsets
+        self.rows = None  # the sequences of the last step, in row order
+        self.table_lens = None  # per group, pages of each row already written to `host`
 
 
 class ModelRunner:
@@ -247,27 +254,93 @@ class ModelRunner:
 
     def _graph_step(self, entries: list[StepEntry], key) -> torch.Tensor:
         batch, widths, ctx_bucket = key
-        self._check(entries)
-        order = list(range(len(entries)))
-        meta = self._meta(entries, order, pad_to=batch, table_widths=list(widths))
         g = self._graphs.get(key)
-        if g is None:
-            g = _DecodeGraph(self.runtime.device)
-            g.meta_dev = torch.zeros(meta.total, dtype=torch.int32, device=self.runtime.device)
-            self._upload(meta, g.meta_dev)
-            g.ctx = self._context(meta, g.meta_dev, g.workspace, max_decode_ctx=ctx_bucket)
-            # once eagerly: every workspace buffer exists before the capture starts
-            self.model.forward(g.ctx, self.layer_caches)
-            torch.cuda.synchronize(self.runtime.device)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                g.logits = self.model.forward(g.ctx, self.layer_caches)
-            g.graph = graph
-            self._graphs[key] = g
-        self._upload(meta, g.meta_dev)
+        if g is None or not self._refresh(g, entries, widths):
+            self._check(entries)
+            order = list(range(len(entries)))
+            meta = self._meta(entries, order, pad_to=batch, table_widths=list(widths))
+            if g is None:
+                g = _DecodeGraph(self.runtime.device)
+                g.meta_dev = torch.zeros(meta.total, dtype=torch.int32, device=self.runtime.device)
+                g.pinned = torch.empty(meta.total, dtype=torch.int32, pin_memory=True)
+                g.host = g.pinned.numpy()
+                g.copied = torch.cuda.Event()
+                offsets, off = {}, 0
+                for name, size in zip(meta.FIELDS, meta.sizes):
+                    offsets[name] = off
+                    off += size
+                offsets["tables"] = []
+                for t in meta.tables:
+                    offsets["tables"].append(off)
+                    off += t.size
+                g.offsets = offsets
+                self._fill(g, entries, meta)
+                g.meta_dev.copy_(g.pinned, non_blocking=True)  # the eager run below reads it
+                g.copied.record()
+                g.ctx = self._context(meta, g.meta_dev, g.workspace, max_decode_ctx=ctx_bucket)
+                # once eagerly: every workspace buffer exists before the capture starts
+                self.model.forward(g.ctx, self.layer_caches)
+                torch.cuda.synchronize(self.runtime.device)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    g.logits = self.model.forward(g.ctx, self.layer_caches)
+                g.graph = graph
+                self._graphs[key] = g
+            else:
+                self._fill(g, entries, meta)
+        g.meta_dev.copy_(g.pinned, non_blocking=True)
+        g.copied.record()
         g.graph.replay()
         self.graph_replays += 1
         return g.logits[: len(entries)]
+
+    def _fill(self, g: _DecodeGraph, entries: list[StepEntry], meta: _Meta) -> None:
+        """Writes a step's whole metadata into the graph's host buffer."""
+        g.copied.synchronize()
+        np.concatenate(meta.parts, out=g.host, casting="unsafe")
+        g.rows = [e.cache for e in entries]  # the objects, so that their identity cannot be reused
+        g.table_lens = [[len(e.cache.tables[gi]) for e in entries]
+                        for gi in range(len(self.cache.groups))]
+
+    def _refresh(self, g: _DecodeGraph, entries: list[StepEntry], widths) -> bool:
+        """The common case of decoding: the same sequences as in the graph's last
+        step, each one token further.  Only what changed is written into the host
+        buffer: tokens, positions, lengths and the pages that were appended.
+        False: the rows differ, and the caller rebuilds the buffer."""
+        if g.rows is None or len(g.rows) != len(entries):
+            return False
+        for e, row in zip(entries, g.rows):
+            if e.cache is not row:
+                return False
+        n = len(entries)
+        tokens = [e.tokens[0] for e in entries]
+        starts = [e.start for e in entries]
+        if min(tokens) < 0 or max(tokens) >= self.vocab_size or min(starts) < 0:
+            return False  # let the full path raise the proper error
+        ps, num_pages = self.cache.page_size, self.cache.num_pages
+        g.copied.synchronize()
+        host, off = g.host, g.offsets
+        # (entries of pages that a window has passed stay as they were: no kernel reads them)
+        for gi in range(len(self.cache.groups)):
+            lens, width, base = g.table_lens[gi], widths[gi], off["tables"][gi]
+            for k, e in enumerate(entries):
+                table = e.cache.tables[gi]
+                have = len(table)
+                if have <= e.start // ps or have > width or have < lens[k]:
+                    return False
+                if have != lens[k]:
+                    new = table[lens[k]:have]
+                    if min(new) < 0 or max(new) >= num_pages:
+                        return False
+                    host[base + k * width + lens[k] : base + k * width + have] = new
+                    lens[k] = have
+        host[off["token_ids"] : off["token_ids"] + n] = tokens
+        host[off["positions"] : off["positions"] + n] = starts
+        ctx = off["ctx_lens"]
+        host[ctx : ctx + n] = starts
+        host[ctx : ctx + n] += 1
+        host[off["fresh"] : off["fresh"] + n] = 0
+        return True
 
     # -------------------------------------------------------------------- step
 
