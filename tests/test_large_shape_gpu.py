@@ -1,0 +1,90 @@
+"""The layer sizes of the Qwen2.5-7B shape (hidden 3584, 28 query heads over 4
+key/value heads of 128, intermediate 18944, vocabulary 152064) with one layer
+and seeded random weights, against the plain implementation: the kernels that
+serving uses at their real sizes (split products, 7 heads per group, a
+vocabulary that is no power of two), in float32 and in bfloat16, cut four ways."""
+
+import random
+
+import pytest
+import torch
+
+from .plain.model import PlainModel, rel_err
+
+pytestmark = pytest.mark.gpu
+
+SHAPE = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "hidden_size": 3584,
+    "intermediate_size": 18944,
+    "num_hidden_layers": 1,
+    "num_attention_heads": 28,
+    "num_key_value_heads": 4,
+    "vocab_size": 152064,
+    "rope_theta": 1000000.0,
+    "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": False,
+    "torch_dtype": "bfloat16",
+}
+
+
+@pytest.fixture(scope="module")
+def model_dir(tmp_path_factory):
+    from shrike_amd.weights import write_model_folder
+
+    return write_model_folder(dict(SHAPE), tmp_path_factory.mktemp("big") / "m", seed=7, mode="unit")
+
+
+@pytest.fixture(scope="module")
+def reference(model_dir):
+    rng = random.Random(5)
+    ids = [rng.randrange(SHAPE["vocab_size"]) for _ in range(150)]
+    plain = PlainModel(model_dir, dtype=torch.float32)  # float64 weights would not fit comfortably
+    want = plain.logits(ids).double()
+    return ids, want
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_one_layer_of_the_7b_shape(dtype, tol, model_dir, reference):
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    ids, want = reference
+    model, rt, _ = load_model(model_dir, dtype)
+    cache = CacheManager(model.cache_specs(), 16, 24, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    runner = ModelRunner(model, cache, rt)
+
+    def run(cuts, other=None):
+        seq = cache.new_sequence()
+        rows, p = [], 0
+        for n in cuts:
+            cache.append(seq, p, n)
+            entries = [StepEntry(seq, ids[p : p + n], p, list(range(n)))]
+            if other is not None:  # another request's single token rides along
+                o, op = other
+                cache.append(o, op[0], 1)
+                entries.insert(0, StepEntry(o, [ids[op[0]]], op[0], [0]))
+                op[0] += 1
+            out = runner.step(entries).cpu()
+            rows.append(out[-n:].clone())
+            p += n
+        cache.free(seq)
+        return torch.cat(rows).double()
+
+    n = len(ids)
+    whole = run([n])
+    assert rel_err(whole, want) <= tol
+    tail = run([n - 32] + [1] * 32)  # the last 32 tokens one by one (graph replays)
+    assert rel_err(tail, want) <= tol
+    portions = run([70, 2, 17, 33, 5, 23])
+    assert rel_err(portions, want) <= tol
+    rider = cache.new_sequence()
+    mixed = run([64, 40, 2, 44], other=(rider, [0]))
+    cache.free(rider)
+    assert rel_err(mixed, want) <= tol
+    if dtype == "float32":
+        for other in (tail, portions, mixed):
+            assert rel_err(other, whole) <= 1e-5
+    cache.check([])
