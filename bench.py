@@ -2,8 +2,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
 
-The model has the layer sizes of the Qwen2.5-7B shape (BASELINE.json
-configs[2]) with random weights in bfloat16.  A "step" is one decode step of
+The model has the layer sizes of the Qwen2.5-7B shape (28 layers, hidden 3584,
+28 query heads over 4 key/value heads of 128, intermediate 18944, vocabulary
+152064) with random weights in bfloat16.  A "step" is one decode step of
 the whole serving path (LLMEngine.step: schedule, forward from the paged cache,
 sample, book-keeping) for `batch` requests that were each prefilled with 2,048
 random tokens; decoding runs towards context 4,096.  One JSON line is printed:
@@ -25,7 +26,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
-# Qwen2.5-7B shape: BASELINE.json configs[2]
+# Qwen2.5-7B shape
 SHAPE_7B = {
     "architectures": ["Qwen2ForCausalLM"],
     "hidden_size": 3584,
