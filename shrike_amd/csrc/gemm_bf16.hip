@@ -60,7 +60,8 @@ __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); 
 template <int NB, int RB>
 __device__ __forceinline__ void skinny_load(SkinnyBatch<NB, RB>& b, const uint4* __restrict__ wrow,
                                             const bf16* __restrict__ a, int lda, int n, int k,
-                                            int ktiles, int t, int step, int j, int kg, bool vec) {
+                                            int ktiles, int t, int step, int j, int kg, bool vec,
+                                            int blocks) {
 #pragma unroll
   for (int u = 0; u < kSkinnyBatch; ++u) {
     const int tt = t + u * step;
@@ -69,7 +70,7 @@ __device__ __forceinline__ void skinny_load(SkinnyBatch<NB, RB>& b, const uint4*
       b.w[u][rb].u = make_uint4(0, 0, 0, 0);
       // weights are read once: a non-temporal load keeps them from displacing
       // the activations in the caches
-      if (tt < ktiles) {
+      if (tt < ktiles && rb < blocks) {
         const uint4* p = wrow + (static_cast<size_t>(rb) * ktiles + tt) * kWave;
         b.w[u][rb].u.x = __builtin_nontemporal_load(&p->x);
         b.w[u][rb].u.y = __builtin_nontemporal_load(&p->y);
@@ -90,23 +91,30 @@ __device__ __forceinline__ void skinny_load(SkinnyBatch<NB, RB>& b, const uint4*
 // one is multiplied.  The host picks WAVES so that about 4096 wavefronts or
 // more are in flight whatever the number of rows.
 //
-// GATED: the weight holds a gated feed-forward's two matrices interleaved by
-// blocks of 16 rows (block 2b: rows 16b.. of the gate matrix, block 2b+1: the
+// MODE kGated: the weight holds a gated feed-forward's two matrices interleaved
+// by blocks of 16 rows (block 2b: rows 16b.. of the gate matrix, block 2b+1: the
 // same rows of the up matrix).  A workgroup multiplies both blocks and writes
 // silu(gate) * up: out[token][16b + row], `m` being the width of that output.
-template <int NB, int WAVES, bool GATED>
+// MODE kPair: a workgroup owns two consecutive blocks of rows, so that every
+// activation it loads feeds two multiplications.
+constexpr int kSingle = 0, kGated = 1, kPair = 2;
+
+template <int NB, int WAVES, int MODE>
 __global__ void __launch_bounds__(WAVES* kWave)
     gemm_skinny_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                        const uint4* __restrict__ wt, int ktiles, int m,
                        const float* __restrict__ bias, void* __restrict__ out, int ldo,
                        int out_f32, int accumulate, int vec, int ksplit) {
-  constexpr int RB = GATED ? 2 : 1;
+  constexpr bool GATED = MODE == kGated;
+  constexpr int RB = MODE == kSingle ? 1 : 2;
   __shared__ float red[WAVES][RB][NB][kWave][4];
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int mb = blockIdx.x;  // block of 16 output rows
+  const int mb = blockIdx.x;  // block of 16 output rows (kPair: of 32)
   const int z = blockIdx.y;   // which share of k (ksplit workgroups per block)
   const int j = lane % 16, kg = lane / 16;
   const uint4* wrow = wt + static_cast<size_t>(mb) * RB * ktiles * kWave + lane;
+  // weight blocks of 16 rows that exist for this workgroup (the last pair may be half)
+  const int blocks = MODE == kPair ? ((m + 15) / 16 - mb * 2 >= 2 ? 2 : 1) : RB;
 
   f32x4 acc[RB][NB];
 #pragma unroll
@@ -119,10 +127,11 @@ __global__ void __launch_bounds__(WAVES* kWave)
   const int lanes_k = WAVES * ksplit;  // wavefronts that share the block's k-tiles
   const int kStride = kSkinnyBatch * lanes_k;
   const int t0 = z * WAVES + wave;
-  skinny_load<NB, RB>(cur, wrow, a, lda, n, k, ktiles, t0, lanes_k, j, kg, vec);
+  skinny_load<NB, RB>(cur, wrow, a, lda, n, k, ktiles, t0, lanes_k, j, kg, vec, blocks);
   for (int t = t0; t < ktiles; t += kStride) {
     if (t + kStride < ktiles)
-      skinny_load<NB, RB>(next, wrow, a, lda, n, k, ktiles, t + kStride, lanes_k, j, kg, vec);
+      skinny_load<NB, RB>(next, wrow, a, lda, n, k, ktiles, t + kStride, lanes_k, j, kg, vec,
+                          blocks);
 #pragma unroll
     for (int u = 0; u < kSkinnyBatch; ++u)
 #pragma unroll
@@ -145,13 +154,15 @@ __global__ void __launch_bounds__(WAVES* kWave)
   // Element e of the block's 16 x (16 * NB) outputs: accumulator b = e / 256,
   // lane (e % 256) / 4, register r = e % 4.  Lane (j, kg) holds rows kg*4 + r
   // for token b*16 + j.  The wavefronts' partial sums are added in wavefront order.
-  for (int e = threadIdx.x; e < NB * 256; e += WAVES * kWave) {
-    const int b = e / 256, ln = (e % 256) / 4, r = e % 4;
-    const int token = b * 16 + ln % 16, row = mb * 16 + (ln / 16) * 4 + r;
+  constexpr int kOutBlocks = MODE == kPair ? 2 : 1;  // blocks of output rows per workgroup
+  for (int e = threadIdx.x; e < kOutBlocks * NB * 256; e += WAVES * kWave) {
+    const int ob = e / (NB * 256), b = (e / 256) % NB, ln = (e % 256) / 4, r = e % 4;
+    const int token = b * 16 + ln % 16;
+    const int row = (mb * kOutBlocks + ob) * 16 + (ln / 16) * 4 + r;
     if (token >= n || row >= m) continue;
-    float v = red[0][0][b][ln][r], up = 0.f;
+    float v = red[0][ob][b][ln][r], up = 0.f;
 #pragma unroll
-    for (int w = 1; w < WAVES; ++w) v += red[w][0][b][ln][r];
+    for (int w = 1; w < WAVES; ++w) v += red[w][ob][b][ln][r];
     if (ksplit > 1) {
       // this workgroup's share of k: a float32 partial sum, [ksplit][n][m], that the
       // kernel which reads the product adds up in order
@@ -334,21 +345,24 @@ __global__ void __launch_bounds__(WAVES* kWave)
 // double-buffered: the loads of stage t+1 are in flight while stage t is
 // multiplied.
 
-// WM x WN: MFMA tiles (16 x 16) per wavefront; the workgroup's 2 x 2 wavefronts
-// cover 32*WM weight rows x 32*WN tokens.  KS: MFMA steps (32 of k) per stage.
-template <int WM, int WN, int KS, bool GATED>
-__global__ void __launch_bounds__(256)
+// GM x GN wavefronts per workgroup, each with WM x WN MFMA tiles (16 x 16): the
+// workgroup covers 16*GM*WM weight rows x 16*GN*WN tokens.  KS: MFMA steps (32 of
+// k) per stage.  The stages live in dynamic LDS, [buffer][fragment][lane].
+template <int GM, int GN, int WM, int WN, int KS, bool GATED>
+__global__ void __launch_bounds__(GM* GN* kWave)
     gemm_big_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                     const uint4* __restrict__ wt, int ktiles, int m,
                     const float* __restrict__ bias, void* __restrict__ out, int ldo, int out_f32,
                     int accumulate, int vec) {
-  constexpr int kWFrags = 2 * WM * KS, kAFrags = 2 * WN * KS;  // fragments per stage
-  // [buffer][fragment][lane]: weights first, then activations
-  __shared__ uint4 stage[2][kWFrags + kAFrags][kWave];
+  constexpr int kWaves = GM * GN;
+  constexpr int kWFrags = GM * WM * KS, kAFrags = GN * WN * KS;  // fragments per stage
+  constexpr int kFrags = kWFrags + kAFrags;
+  extern __shared__ uint4 stage_mem[];
+  auto stage = [&](int buf, int frag) -> uint4* { return stage_mem + (buf * kFrags + frag) * kWave; };
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int wm = wave / 2, wn = wave % 2;  // quadrant of the wavefront
-  const int mb0 = blockIdx.x * (2 * WM);   // first block of 16 weight rows
-  const int tok0 = blockIdx.y * (32 * WN);
+  const int wm = wave / GN, wn = wave % GN;  // place of the wavefront in the workgroup's tile
+  const int mb0 = blockIdx.x * (GM * WM);  // first block of 16 weight rows
+  const int tok0 = blockIdx.y * (16 * GN * WN);
   // blocks of 16 weight rows; a gated weight has two per 16 output rows
   const int mblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
   const int nstages = (ktiles + KS - 1) / KS;
@@ -360,20 +374,20 @@ __global__ void __launch_bounds__(256)
     for (int jn = 0; jn < WN; ++jn) acc[i][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // Fragment f of an operand is (block of 16 rows f / KS, MFMA step f % KS); wavefront w
-  // moves fragments w, w + 4, ...
-  constexpr int kWPer = (kWFrags + 3) / 4, kAPer = (kAFrags + 3) / 4;
+  // moves fragments w, w + kWaves, ...
+  constexpr int kWPer = (kWFrags + kWaves - 1) / kWaves, kAPer = (kAFrags + kWaves - 1) / kWaves;
   uint4 wreg[kWPer], areg[kAPer];
   auto load_stage = [&](int st) {
 #pragma unroll
     for (int i = 0; i < kWPer; ++i) {
-      const int f = wave + 4 * i, rb = f / KS, kt = st * KS + f % KS;
+      const int f = wave + kWaves * i, rb = f / KS, kt = st * KS + f % KS;
       wreg[i] = make_uint4(0, 0, 0, 0);
       if (f < kWFrags && mb0 + rb < mblocks && kt < ktiles)
         wreg[i] = wt[(static_cast<size_t>(mb0 + rb) * ktiles + kt) * kWave + lane];
     }
 #pragma unroll
     for (int i = 0; i < kAPer; ++i) {
-      const int f = wave + 4 * i, rb = f / KS, kt = st * KS + f % KS;
+      const int f = wave + kWaves * i, rb = f / KS, kt = st * KS + f % KS;
       areg[i] = make_uint4(0, 0, 0, 0);
       if (f < kAFrags)
         areg[i] = load_act(a, lda, n, k, tok0 + rb * 16 + lane % 16, kt * 32 + (lane / 16) * 8, vec).u;
@@ -382,10 +396,10 @@ __global__ void __launch_bounds__(256)
   auto store_stage = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < kWPer; ++i)
-      if (wave + 4 * i < kWFrags) stage[buf][wave + 4 * i][lane] = wreg[i];
+      if (wave + kWaves * i < kWFrags) stage(buf, wave + kWaves * i)[lane] = wreg[i];
 #pragma unroll
     for (int i = 0; i < kAPer; ++i)
-      if (wave + 4 * i < kAFrags) stage[buf][kWFrags + wave + 4 * i][lane] = areg[i];
+      if (wave + kWaves * i < kAFrags) stage(buf, kWFrags + wave + kWaves * i)[lane] = areg[i];
   };
 
   load_stage(0);
@@ -398,11 +412,11 @@ __global__ void __launch_bounds__(256)
     for (int ks = 0; ks < KS; ++ks) {
       Frag af[WN];
 #pragma unroll
-      for (int jn = 0; jn < WN; ++jn) af[jn].u = stage[buf][kWFrags + (wn * WN + jn) * KS + ks][lane];
+      for (int jn = 0; jn < WN; ++jn) af[jn].u = stage(buf, kWFrags + (wn * WN + jn) * KS + ks)[lane];
 #pragma unroll
       for (int i = 0; i < WM; ++i) {
         Frag wf;
-        wf.u = stage[buf][(wm * WM + i) * KS + ks][lane];
+        wf.u = stage(buf, (wm * WM + i) * KS + ks)[lane];
 #pragma unroll
         for (int jn = 0; jn < WN; ++jn)
           acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, af[jn].v, acc[i][jn], 0, 0, 0);
@@ -548,31 +562,37 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   if (n > 64) {
     SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
     const int wblocks = (gated ? 2 : 1) * mb;  // blocks of 16 weight rows
-#define SHK_BIG(WM, WN, KS)                                                                  \
-  do {                                                                                       \
-    dim3 grid((wblocks + 2 * WM - 1) / (2 * WM), (n + 32 * WN - 1) / (32 * WN));            \
-    SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);                        \
-    if (gated)                                                                               \
-      gemm_big_kernel<WM, WN, KS, true><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, \
-                                                             out, ldo, of, accumulate, vec); \
-    else                                                                                     \
-      gemm_big_kernel<WM, WN, KS, false><<<grid, 256, 0, s>>>(ap, lda, n, k, wp, kt, m, bias, \
-                                                              out, ldo, of, accumulate, vec); \
+#define SHK_BIG(GM, GN, WM, WN, KS)                                                            \
+  do {                                                                                         \
+    constexpr int lds = 2 * (GM * WM + GN * WN) * KS * kWave * 16;                             \
+    dim3 grid((wblocks + GM * WM - 1) / (GM * WM), (n + 16 * GN * WN - 1) / (16 * GN * WN));   \
+    SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);                          \
+    if (gated) {                                                                               \
+      auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, true>;                                 \
+      if (lds > 65536)                                                                         \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                             \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);                  \
+      kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,  \
+                                                accumulate, vec);                              \
+    } else {                                                                                   \
+      auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, false>;                                \
+      if (lds > 65536)                                                                         \
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                             \
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);                  \
+      kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,  \
+                                                accumulate, vec);                              \
+    }                                                                                          \
   } while (0)
-    // 128 x 128 per workgroup, 64 of k per stage.  (Tiles of 256 rows measured slower:
-    // their accumulators no longer fit the register file.)
-    SHK_BIG(4, 4, 2);
+    // 128 x 128 per workgroup, 64 of k per stage (128 x 256 with eight wavefronts
+    // measured slower: the staging, not the arithmetic, bounds this kernel)
+    SHK_BIG(2, 2, 4, 4, 2);
 #undef SHK_BIG
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }
   if (n > 16) {
     // blocks of output rows per workgroup: 8 where that still leaves enough workgroups
-#ifdef SHK_MID_WAVES
-    const int mid_waves = (mb >= 4096) ? 8 : SHK_MID_WAVES;
-#else
     const int mid_waves = (mb >= 4096) ? 8 : 4;
-#endif
     dim3 mgrid((mb + mid_waves - 1) / mid_waves, ksplit);
 #define SHK_MID_W(NB, W)                                                                    \
   do {                                                                                      \
@@ -587,8 +607,6 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   do {                       \
     if (mid_waves == 8)      \
       SHK_MID_W(NB, 8);      \
-    else if (mid_waves == 2) \
-      SHK_MID_W(NB, 2);      \
     else                     \
       SHK_MID_W(NB, 4);      \
   } while (0)
@@ -603,14 +621,20 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   // wavefronts per workgroup: matrices with few row blocks get more of them
   const int waves = (mb >= 512 || ksplit > 1) ? ((mb >= 512) ? 8 : 4) : 16;
   const int max_waves = 16;
-  dim3 sgrid(mb, ksplit);
+  // two row blocks per workgroup share their activation loads, where the matrix has
+  // enough blocks to fill the chip with half as many workgroups
+  const bool pair = !gated && mb >= 128;
+  dim3 sgrid(pair ? (mb + 1) / 2 : mb, ksplit);
 #define SHK_SKINNY_W(NB, W)                                                                     \
   do {                                                                                          \
     if (gated)                                                                                  \
-      gemm_skinny_kernel<NB, W, true><<<sgrid, W * kWave, 0, s>>>(                              \
+      gemm_skinny_kernel<NB, W, kGated><<<sgrid, W * kWave, 0, s>>>(                            \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);               \
+    else if (pair)                                                                              \
+      gemm_skinny_kernel<NB, W, kPair><<<sgrid, W * kWave, 0, s>>>(                             \
           ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);               \
     else                                                                                        \
-      gemm_skinny_kernel<NB, W, false><<<sgrid, W * kWave, 0, s>>>(                             \
+      gemm_skinny_kernel<NB, W, kSingle><<<sgrid, W * kWave, 0, s>>>(                           \
           ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec, ksplit);               \
   } while (0)
 #define SHK_SKINNY(NB)                       \

@@ -15,10 +15,6 @@ import torch
 
 from ..kernels import ops
 
-import os
-
-_EXPERIMENT_TILE_KERNEL = bool(os.environ.get("SHRIKE_PREFILL_TILE"))
-
 
 class LinearWeight:
     """A weight matrix [rows, cols] as the kernels want it."""
@@ -102,8 +98,6 @@ class Runtime:
                                      cache.k_pool, cache.v_pool, cache.page_size, spec.window,
                                      spec.scale, partial, nsplit)
             tiles = ops.attention_prefill_shared_tiles(h, hkv, d) if ctx.num_prefill_tiles else 0
-            if _EXPERIMENT_TILE_KERNEL:
-                tiles = 0
             if tiles:
                 wg_seq, wg_q0, count = ctx.prefill_workgroups(tiles)
                 ops.attention_prefill_shared(q, out, count, h, hkv, d, ctx.cu_q, ctx.ctx_lens, wg_seq,
