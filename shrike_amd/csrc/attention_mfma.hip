@@ -138,197 +138,465 @@ __device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, cons
   }
 }
 
+// One chunk of 32 keys at `kb` for 16 rows: scores, running softmax state,
+// O += P V.  p_lds: this wavefront's 16 x kPStride staging tile.
+template <int D>
+__device__ __forceinline__ void attend_chunk(const TileArgs& ta, const AFrag (&qf)[D / 32],
+                                             const Chunk<D>& cur, int kb, const int (&row_pos)[4],
+                                             const int (&row_lo)[4], int pos_max, int lo_min,
+                                             f32x4 (&o)[D / 16], float (&m)[4], float (&l)[4],
+                                             uint16_t* p_lds) {
+  const int lane = threadIdx.x % kWave;
+  const int j = lane % 16, kg = lane / 16;
+
+  // ---- S = Q K^T for two tiles of 16 keys
+  f32x4 s[2];
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt) {
+    s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ds = 0; ds < D / 32; ++ds)
+      s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ds].v, cur.k[tt][ds].v, s[tt], 0, 0, 0);
+  }
+
+  // ---- mask, running maximum and sum (lane holds key kb + tt*16 + j for rows 4*kg + r)
+  float p[2][4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    float sc[2];
+#pragma unroll
+    for (int tt = 0; tt < 2; ++tt) {
+      const int key = kb + tt * 16 + j;
+      const bool keep = key <= row_pos[r] && key >= row_lo[r];
+      sc[tt] = keep ? s[tt][r] * ta.scale : -INFINITY;
+    }
+    const float mx = row16_max(fmaxf(sc[0], sc[1]));
+    const float m_new = fmaxf(m[r], mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = __expf(m[r] - m_safe);
+    p[0][r] = __expf(sc[0] - m_safe);
+    p[1][r] = __expf(sc[1] - m_safe);
+    const float sum = row16_sum(p[0][r] + p[1][r]);
+    l[r] = l[r] * alpha + sum;
+    m[r] = m_new;
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) o[db][r] *= alpha;
+  }
+
+  // ---- P through LDS into A-operand layout: rows 16, keys 32.  The tile belongs
+  // to this wavefront alone; the fences order its own writes and reads.
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+      p_lds[(kg * 4 + r) * kPStride + tt * 16 + j] = bf16_bits(p[tt][r]);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  AFrag pf;
+  pf.u = *reinterpret_cast<const uint4*>(p_lds + j * kPStride + kg * 8);
+
+  // ---- O += P V.  Keys outside [lo_min, pos_max] carry weight 0 but their
+  // slots may hold anything: zero them so that 0 * x stays 0.
+  const int g0 = kb + kg * 8;
+  uint4 keep_bits = make_uint4(~0u, ~0u, ~0u, ~0u);
+  if (g0 < lo_min || g0 + 7 > pos_max) {
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const bool a = g0 + 2 * e >= lo_min && g0 + 2 * e <= pos_max;
+      const bool b = g0 + 2 * e + 1 >= lo_min && g0 + 2 * e + 1 <= pos_max;
+      w[e] = (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
+    }
+    keep_bits = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) {
+    AFrag vf = cur.v[db];
+    vf.u.x &= keep_bits.x;
+    vf.u.y &= keep_bits.y;
+    vf.u.z &= keep_bits.z;
+    vf.u.w &= keep_bits.w;
+    o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, o[db], 0, 0, 0);
+  }
+}
+
 // Walks keys [key_begin, key_end) (key_begin a multiple of 32) for 16 rows.
 // qf: the rows' queries as A operands.  row_pos / row_lo: for this lane's four
 // accumulator rows (4*(lane/16) + r), the last and first key each may read.
-// pos_max / lo_min: the same bounds over all 16 rows.  The next chunk's loads
+// pos_max / lo_min: the same bounds over all 16 rows.  NBUF - 1 chunks' loads
 // are in flight while the current chunk is computed.
-template <int D>
+template <int D, int NBUF = 2>
 __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf)[D / 32],
                                             const int (&row_pos)[4], const int (&row_lo)[4],
                                             int pos_max, int lo_min, int key_begin, int key_end,
                                             f32x4 (&o)[D / 16], float (&m)[4], float (&l)[4],
                                             uint16_t* p_lds) {
-  const int lane = threadIdx.x % kWave;
-  const int j = lane % 16, kg = lane / 16;
-
   const int ps = ta.page_size;
   const int last_entry = pos_max / ps;
   PageWindow pw = load_pages(ta.table, key_begin / ps, last_entry);
-  Chunk<D> cur, nxt;
-  if (key_begin < key_end) load_chunk<D>(cur, ta, pw, key_begin, pos_max, lo_min);
-  for (int kb = key_begin; kb < key_end; kb += 32) {
-    if (kb + 32 < key_end) {
-      // the window must hold the entries of keys kb + 32 .. kb + 63
-      if ((kb + 63) / ps >= pw.base + kWave) pw = load_pages(ta.table, (kb + 32) / ps, last_entry);
-      load_chunk<D>(nxt, ta, pw, kb + 32, pos_max, lo_min);
-    }
-
-    // ---- S = Q K^T for two tiles of 16 keys
-    f32x4 s[2];
+  Chunk<D> buf[NBUF];
+  // the window must hold the entries of the 32 keys from `kb` before they are loaded
+  auto fetch = [&](Chunk<D>& c, int kb) {
+    if ((kb + 31) / ps >= pw.base + kWave) pw = load_pages(ta.table, kb / ps, last_entry);
+    load_chunk<D>(c, ta, pw, kb, pos_max, lo_min);
+  };
 #pragma unroll
-    for (int tt = 0; tt < 2; ++tt) {
-      s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int u = 0; u < NBUF - 1; ++u)
+    if (key_begin + 32 * u < key_end) fetch(buf[u], key_begin + 32 * u);
+  for (int kb0 = key_begin; kb0 < key_end; kb0 += 32 * NBUF) {
 #pragma unroll
-      for (int ds = 0; ds < D / 32; ++ds)
-        s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ds].v, cur.k[tt][ds].v, s[tt], 0, 0, 0);
-    }
-
-    // ---- mask, running maximum and sum (lane holds key kb + tt*16 + j for rows 4*kg + r)
-    float p[2][4];
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      float sc[2];
-#pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        const int key = kb + tt * 16 + j;
-        const bool keep = key <= row_pos[r] && key >= row_lo[r];
-        sc[tt] = keep ? s[tt][r] * ta.scale : -INFINITY;
+    for (int u = 0; u < NBUF; ++u) {
+      const int kb = kb0 + 32 * u;
+      if (kb < key_end) {
+        const int ahead = kb + 32 * (NBUF - 1);
+        if (ahead < key_end) fetch(buf[(u + NBUF - 1) % NBUF], ahead);
+        attend_chunk<D>(ta, qf, buf[u], kb, row_pos, row_lo, pos_max, lo_min, o, m, l, p_lds);
       }
-      const float mx = row16_max(fmaxf(sc[0], sc[1]));
-      const float m_new = fmaxf(m[r], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __expf(m[r] - m_safe);
-      p[0][r] = __expf(sc[0] - m_safe);
-      p[1][r] = __expf(sc[1] - m_safe);
-      const float sum = row16_sum(p[0][r] + p[1][r]);
-      l[r] = l[r] * alpha + sum;
-      m[r] = m_new;
-#pragma unroll
-      for (int db = 0; db < D / 16; ++db) o[db][r] *= alpha;
     }
-
-    // ---- P through LDS into A-operand layout: rows 16, keys 32
-    __syncthreads();  // the previous chunk's reads are done (one wavefront per workgroup)
-#pragma unroll
-    for (int tt = 0; tt < 2; ++tt)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        p_lds[(kg * 4 + r) * kPStride + tt * 16 + j] = bf16_bits(p[tt][r]);
-    __syncthreads();
-    AFrag pf;
-    pf.u = *reinterpret_cast<const uint4*>(p_lds + j * kPStride + kg * 8);
-
-    // ---- O += P V.  Keys outside [lo_min, pos_max] carry weight 0 but their
-    // slots may hold anything: zero them so that 0 * x stays 0.
-    const int g0 = kb + kg * 8;
-    uint4 keep_bits = make_uint4(~0u, ~0u, ~0u, ~0u);
-    if (g0 < lo_min || g0 + 7 > pos_max) {
-      uint32_t w[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const bool a = g0 + 2 * e >= lo_min && g0 + 2 * e <= pos_max;
-        const bool b = g0 + 2 * e + 1 >= lo_min && g0 + 2 * e + 1 <= pos_max;
-        w[e] = (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
-      }
-      keep_bits = make_uint4(w[0], w[1], w[2], w[3]);
-    }
-#pragma unroll
-    for (int db = 0; db < D / 16; ++db) {
-      AFrag vf = cur.v[db];
-      vf.u.x &= keep_bits.x;
-      vf.u.y &= keep_bits.y;
-      vf.u.z &= keep_bits.z;
-      vf.u.w &= keep_bits.w;
-      o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, o[db], 0, 0, 0);
-    }
-    cur = nxt;
   }
 }
 
 // ------------------------------------------------------------------- decode
-// grid (kv_heads, sequences, splits), one wavefront per workgroup.
+// grid (kv_heads, sequences, splits), kDecodeWaves wavefronts per workgroup.  A
+// single wavefront needs about 1,700 cycles for a chunk of 32 keys whatever the
+// memory does, so a workgroup's key range is dealt out to its wavefronts chunk
+// by chunk, and their results are combined through LDS before anything is
+// written.
+//
+// The two products are formed transposed, so that a lane owns one query head
+// throughout and nothing passes through LDS:
+//   S^T = K Q^T   A = 16 keys x head_dim, B = Q^T.  Row i of the A tile t is key
+//                 8*(i/4) + 4*t + i%4 of the chunk, so lane (j, g) ends up with
+//                 the scores of query j for the eight keys 8*g .. 8*g + 7;
+//   O^T += V^T P^T  those eight probabilities, packed to bfloat16, are lane
+//                 (j, g)'s B operand as they stand; A is V^T (8 keys of one
+//                 element: one 16-byte load from the transposed page).
+// Keys outside [lo, pos] are loaded from a slot of a page the sequence holds
+// (the page of the nearest key inside the range) and masked.
+
+constexpr int kMaxSplits = 64;
+constexpr int kDecodeWaves = 4;
+
+template <bool V>
+struct EdgeTag {
+  static constexpr bool value = V;
+};
 
 template <int D>
-__global__ void __launch_bounds__(kWave)
-    attention_decode_kernel(const bf16* __restrict__ q, int q_stride, int heads, int kv_heads,
-                            const int32_t* __restrict__ positions,
+struct DecodeChunk {
+  AFrag k[2][D / 32];
+  AFrag v[D / 16];
+};
+
+// x / page_size and x % page_size without a division: magic = ceil(2^32 / page_size)
+// makes the high half of x * magic the quotient for 0 <= x < 2^32 / page_size.
+struct PageDiv {
+  int ps;
+  uint32_t magic;
+  __device__ __forceinline__ int div(int x) const {
+    return static_cast<int>(__umulhi(static_cast<uint32_t>(x), magic));
+  }
+  __device__ __forceinline__ int mod(int x) const { return x - div(x) * ps; }
+};
+
+template <int D>
+__global__ void __launch_bounds__(kDecodeWaves* kWave)
+    attention_decode_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
+                            int heads, int kv_heads, const int32_t* __restrict__ positions,
                             const int32_t* __restrict__ tables, int table_stride,
                             const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
-                            int page_size, int window, float scale, float* __restrict__ partial,
-                            int nsplit) {
-  __shared__ __attribute__((aligned(16))) uint16_t p_lds[16 * kPStride];
+                            int page_size, uint32_t page_magic, int window, float scale,
+                            float* __restrict__ partial, int nsplit) {
+  constexpr int NBUF = 2;  // chunk buffers: one computed, one in flight
+  constexpr int kStep = 32 * kDecodeWaves;  // keys between two chunks of one wavefront
+  __shared__ float m_lds[kDecodeWaves][16], l_lds[kDecodeWaves][16];
+  __shared__ float4 o_lds[kDecodeWaves - 1][D / 16][kWave];
   const int kvh = blockIdx.x, seq = blockIdx.y, z = blockIdx.z;
-  const int lane = threadIdx.x, j = lane % 16, kg = lane / 16;
+  const int wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x % kWave, j = lane % 16, g = lane / 16;
   const int group = heads / kv_heads;
+  const PageDiv pd{page_size, page_magic};
   // decode sequences come first in the step: token index == sequence index
   const int pos = positions[seq];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
 
-  // this split's keys: chunks of 32 from the chunk that holds `lo`
+  // this split's keys: chunks of 32 from the chunk that holds `lo`; this
+  // wavefront's chunks are those at key_begin, key_begin + kStep, ...
   const int first = lo & ~31;
   const int chunks = (pos - first) / 32 + 1;
   const int per = (chunks + nsplit - 1) / nsplit;
-  const int key_begin = first + z * per * 32;
-  int key_end = key_begin + per * 32;
+  const int key_begin = first + z * per * 32 + wave * 32;
+  int key_end = first + (z + 1) * per * 32;
   if (key_end > pos + 1) key_end = pos + 1;
 
-  float m[4], l[4];
-  f32x4 o[D / 16];
-#pragma unroll
-  for (int r = 0; r < 4; ++r) m[r] = -INFINITY, l[r] = 0.f;
+  // softmax state of query head j in base-2 logarithms; `l` is this lane's share
+  // of the sum (its eight keys of every chunk) until the end
+  float m = -INFINITY, l = 0.f;
+  f32x4 o[D / 16];  // element db*16 + 4*g + r of query j
 #pragma unroll
   for (int db = 0; db < D / 16; ++db) o[db] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  if (key_begin <= pos) {
+  if (key_begin < key_end) {
     AFrag qf[D / 32];
     const bf16* qrow = q + static_cast<size_t>(seq) * q_stride +
-                       static_cast<size_t>(kvh * group + j) * D + kg * 8;
+                       static_cast<size_t>(kvh * group + j) * D + g * 8;
 #pragma unroll
     for (int ds = 0; ds < D / 32; ++ds) {
       qf[ds].u = make_uint4(0, 0, 0, 0);
       if (j < group) qf[ds].u = *reinterpret_cast<const uint4*>(qrow + ds * 32);
     }
-    const int row_pos[4] = {pos, pos, pos, pos};
-    const int row_lo[4] = {lo, lo, lo, lo};
-    TileArgs ta{tables + static_cast<size_t>(seq) * table_stride, k_pool, v_pool, page_size,
-                kv_heads, kvh, scale};
-    attend_tile<D>(ta, qf, row_pos, row_lo, pos, lo, key_begin, key_end, o, m, l, p_lds);
-  }
+    const float scale2 = scale * 1.4426950408889634f;
+    const int32_t* table = tables + static_cast<size_t>(seq) * table_stride;
+    // what of a load's address belongs to the lane: its row inside a half chunk
+    // of 16 keys and whether it reads the first or the second half
+    const bool k_second = j >= 8;
+    int k_lane[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) k_lane[t] = (8 * ((j / 4) % 2) + 4 * t + j % 4) * D + g * 8;
+    const bool v_second = g >= 2;
+    const int v_lane = j * page_size + 8 * (g % 2);
+    const size_t head_elems = static_cast<size_t>(page_size) * D;  // one kv head of one page
 
-  // partial[seq][head][split] = {O[D], max, sum}; lane holds element db*16 + j of rows 4*kg + r
+    auto fetch = [&](DecodeChunk<D>& c, int kb) {
+      // pages of the two halves (wave-uniform), clamped into the range the sequence holds
+      int ka = kb < lo ? lo : kb, kc = kb + 16 < lo ? lo : kb + 16;
+      ka = ka > pos ? pos : ka;
+      kc = kc > pos ? pos : kc;
+      // scalar loads: they are counted apart from the vector loads in flight
+      const int page_a = table[__builtin_amdgcn_readfirstlane(pd.div(ka))];
+      const int page_c = table[__builtin_amdgcn_readfirstlane(pd.div(kc))];
+      const size_t head_a = (static_cast<size_t>(page_a) * kv_heads + kvh) * head_elems;
+      const size_t head_c = (static_cast<size_t>(page_c) * kv_heads + kvh) * head_elems;
+      const int slot_a = pd.mod(kb), slot_c = pd.mod(kb + 16);
+      const bf16* krow = k_pool + (k_second ? head_c + static_cast<size_t>(slot_c) * D
+                                            : head_a + static_cast<size_t>(slot_a) * D);
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int hrow = kg * 4 + r;
-    if (hrow >= group) continue;
-    float* dst = partial + ((static_cast<size_t>(seq) * heads + kvh * group + hrow) * nsplit + z) *
-                               (D + 2);
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int db = 0; db < D / 16; ++db) dst[db * 16 + j] = o[db][r];
-    if (j == 0) {
-      dst[D] = m[r];
-      dst[D + 1] = l[r];
+        for (int ds = 0; ds < D / 32; ++ds)
+          c.k[t][ds].u = *reinterpret_cast<const uint4*>(krow + k_lane[t] + ds * 32);
+      const bf16* vcol = v_pool + (v_second ? head_c + slot_c : head_a + slot_a) + v_lane;
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db)
+        c.v[db].u = *reinterpret_cast<const uint4*>(vcol + static_cast<size_t>(db) * 16 * page_size);
+    };
+
+    auto attend_chunk = [&](const DecodeChunk<D>& c, int kb, auto edge_tag) {
+      constexpr bool edge = decltype(edge_tag)::value;
+      f32x4 s[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ds = 0; ds < D / 32; ++ds)
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(c.k[t][ds].v, qf[ds].v, s[t], 0, 0, 0);
+      }
+      // this lane's keys are kb + 8*g + e, e = 4*t + r
+      float sc[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sc[e] = s[e / 4][e % 4] * scale2;
+      const int g0 = kb + g * 8;
+      if (edge) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (g0 + e > pos || g0 + e < lo) sc[e] = -INFINITY;
+      }
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                       fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m, mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
+      float pr[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pr[e] = __builtin_amdgcn_exp2f(sc[e] - m_safe);
+      l = l * alpha + (((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7])));
+      m = m_new;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+        for (int db = 0; db < D / 16; ++db) o[db] *= alpha;
+      }
+      AFrag pf;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pf.v[e] = static_cast<__bf16>(pr[e]);
+      // Masked keys carry weight 0 but their slots may hold anything: zero them
+      // so that 0 * x stays 0.
+      uint4 keep_bits = make_uint4(~0u, ~0u, ~0u, ~0u);
+      if (edge) {
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool a = g0 + 2 * e >= lo && g0 + 2 * e <= pos;
+          const bool b = g0 + 2 * e + 1 >= lo && g0 + 2 * e + 1 <= pos;
+          w[e] = (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
+        }
+        keep_bits = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db) {
+        AFrag vf = c.v[db];
+        if (edge) {
+          vf.u.x &= keep_bits.x;
+          vf.u.y &= keep_bits.y;
+          vf.u.z &= keep_bits.z;
+          vf.u.w &= keep_bits.w;
+        }
+        o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, o[db], 0, 0, 0);
+      }
+    };
+
+    // interior chunks, the common case, carry no masking code
+    auto attend = [&](const DecodeChunk<D>& c, int kb) {
+      if (kb + 31 > pos || kb < lo)  // wave-uniform
+        attend_chunk(c, kb, EdgeTag<true>{});
+      else
+        attend_chunk(c, kb, EdgeTag<false>{});
+    };
+
+    // NBUF - 1 chunks' loads are in flight while one chunk is computed.  Every step
+    // issues a chunk's loads, past the end those of the last chunk again: a step
+    // without loads would make the compiler wait for all loads in flight at each step.
+    const int last_kb = key_begin + (key_end - 1 - key_begin) / kStep * kStep;
+    DecodeChunk<D> buf[NBUF];
+#pragma unroll
+    for (int u = 0; u < NBUF - 1; ++u) {
+      const int kb = key_begin + kStep * u;
+      fetch(buf[u], kb < last_kb ? kb : last_kb);
     }
+    for (int kb0 = key_begin; kb0 < key_end; kb0 += kStep * NBUF) {
+#pragma unroll
+      for (int u = 0; u < NBUF; ++u) {
+        const int kb = kb0 + kStep * u;
+        if (kb >= key_end) break;
+        const int ahead = kb + kStep * (NBUF - 1);
+        fetch(buf[(u + NBUF - 1) % NBUF], ahead < last_kb ? ahead : last_kb);
+        attend(buf[u], kb);
+      }
+    }
+    l += __shfl_xor(l, 16, kWave);
+    l += __shfl_xor(l, 32, kWave);
   }
-}
 
-// out[seq][head][:] = sum_z exp(m_z - M) O_z / sum_z exp(m_z - M) l_z, splits in order.
-constexpr int kMaxSplits = 64;
-
-__global__ void attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out,
-                                       int head_dim, int nsplit) {
-  __shared__ float ms[kMaxSplits], ls[kMaxSplits];
-  const size_t row = blockIdx.x;  // seq * heads + head
-  const int stride = head_dim + 2;
-  const float* src = partial + row * nsplit * stride;
-  if (threadIdx.x < nsplit) {
-    ms[threadIdx.x] = src[threadIdx.x * stride + head_dim];
-    ls[threadIdx.x] = src[threadIdx.x * stride + head_dim + 1];
+  // ---- the wavefronts' results become one: common maximum, sums in wavefront order
+  if (g == 0) {
+    m_lds[wave][j] = m;
+    l_lds[wave][j] = l;
   }
   __syncthreads();
-  float mx = -INFINITY;
-  for (int z = 0; z < nsplit; ++z) mx = fmaxf(mx, ms[z]);
-  float den = 0.f;
-  for (int z = 0; z < nsplit; ++z) den += (ms[z] == -INFINITY ? 0.f : __expf(ms[z] - mx)) * ls[z];
-  const float inv = 1.f / den;
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float num = 0.f;
-#pragma unroll 8
-    for (int z = 0; z < nsplit; ++z) {
-      const float f = ms[z] == -INFINITY ? 0.f : __expf(ms[z] - mx);
-      num += f * src[z * stride + d];
+  float m_all = m_lds[0][j];
+#pragma unroll
+  for (int w = 1; w < kDecodeWaves; ++w) m_all = fmaxf(m_all, m_lds[w][j]);
+  const float m_ref = (m_all == -INFINITY) ? 0.f : m_all;
+  l = 0.f;
+#pragma unroll
+  for (int w = 0; w < kDecodeWaves; ++w)
+    l += l_lds[w][j] * __builtin_amdgcn_exp2f(m_lds[w][j] - m_ref);  // 2^-inf = 0: nothing seen
+  const float mine = __builtin_amdgcn_exp2f(m - m_ref);
+  m = m_all;
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db) o[db] *= mine;
+  if (wave > 0) {
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db)
+      o_lds[wave - 1][db][lane] = make_float4(o[db][0], o[db][1], o[db][2], o[db][3]);
+  }
+  __syncthreads();
+  if (wave > 0 || j >= group) return;
+#pragma unroll
+  for (int w = 0; w < kDecodeWaves - 1; ++w)
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      const float4 x = o_lds[w][db][lane];
+      o[db][0] += x.x;
+      o[db][1] += x.y;
+      o[db][2] += x.z;
+      o[db][3] += x.w;
     }
-    out[row * head_dim + d] = from_float<bf16>(num * inv);
+
+  const int head = kvh * group + j;
+  if (nsplit == 1) {
+    // the whole range in one wavefront: normalise and write the output row
+    const float inv = 1.f / l;
+    bf16* dst = out + (static_cast<size_t>(seq) * heads + head) * D + 4 * g;
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      uint2 packed;
+      packed.x = bf16_bits(o[db][0] * inv) | (static_cast<uint32_t>(bf16_bits(o[db][1] * inv)) << 16);
+      packed.y = bf16_bits(o[db][2] * inv) | (static_cast<uint32_t>(bf16_bits(o[db][3] * inv)) << 16);
+      *reinterpret_cast<uint2*>(dst + db * 16) = packed;
+    }
+    return;
+  }
+  // partial: O [seq][head][split][D], then (max, sum) [seq][head][split][2]
+  const size_t rows = static_cast<size_t>(gridDim.y) * heads * nsplit;
+  const size_t row = (static_cast<size_t>(seq) * heads + head) * nsplit + z;
+  float* dst = partial + row * D + 4 * g;
+#pragma unroll
+  for (int db = 0; db < D / 16; ++db)
+    *reinterpret_cast<float4*>(dst + db * 16) = make_float4(o[db][0], o[db][1], o[db][2], o[db][3]);
+  if (g == 0) *reinterpret_cast<float2*>(partial + rows * D + row * 2) = make_float2(m, l);
+}
+
+// out[seq][head][:] = sum_z 2^(m_z - M) O_z / sum_z 2^(m_z - M) l_z, splits in
+// order.  One wavefront per (sequence, head); lane z holds split z's weight.
+template <int D>
+__global__ void __launch_bounds__(kWave)
+    attention_merge_kernel(const float* __restrict__ partial, bf16* __restrict__ out, int nsplit) {
+  constexpr int NE = (D + kWave - 1) / kWave;  // elements per lane
+  constexpr int kBatch = 8;                    // splits in flight
+  __shared__ float weight[kMaxSplits];
+  const size_t rows = static_cast<size_t>(gridDim.x) * nsplit;
+  const size_t row = blockIdx.x;  // seq * heads + head
+  const int lane = threadIdx.x;
+  const float* src = partial + row * nsplit * D;
+  const float* ml = partial + rows * D + row * nsplit * 2;
+  float2 mine = make_float2(-INFINITY, 0.f);
+  if (lane < nsplit) mine = *reinterpret_cast<const float2*>(ml + lane * 2);
+
+  float x[kBatch][NE];
+  auto fetch = [&](int z0) {
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u)
+#pragma unroll
+      for (int e = 0; e < NE; ++e) {
+        const int d = lane + e * kWave;
+        x[u][e] = (z0 + u < nsplit && d < D) ? src[static_cast<size_t>(z0 + u) * D + d] : 0.f;
+      }
+  };
+  fetch(0);  // travels while the weights are formed
+
+  const float mx = wave_max(mine.x);
+  const float w = mine.x == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mine.x - mx);
+  weight[lane] = w;
+  // splits in order: the denominator is summed by every lane from the weights in LDS
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const float wl = w * mine.y;
+  float den = 0.f;
+  for (int zz = 0; zz < nsplit; ++zz) den += __shfl(wl, zz, kWave);
+
+  float acc[NE];
+#pragma unroll
+  for (int e = 0; e < NE; ++e) acc[e] = 0.f;
+  for (int z0 = 0; z0 < nsplit; z0 += kBatch) {
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const float wz = z0 + u < nsplit ? weight[z0 + u] : 0.f;
+#pragma unroll
+      for (int e = 0; e < NE; ++e) acc[e] += wz * x[u][e];
+    }
+    if (z0 + kBatch < nsplit) fetch(z0 + kBatch);
+  }
+  const float inv = 1.f / den;
+#pragma unroll
+  for (int e = 0; e < NE; ++e) {
+    const int d = lane + e * kWave;
+    if (d < D) out[row * D + d] = from_float<bf16>(acc[e] * inv);
   }
 }
 
@@ -609,13 +877,16 @@ __global__ void __launch_bounds__(kSharedWaves* kWave) __attribute__((amdgpu_wav
 }
 
 template <int D>
-static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, int heads,
-                          int kv_heads, const int32_t* positions, const int32_t* tables,
+static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, bf16* out,
+                          int heads, int kv_heads, const int32_t* positions, const int32_t* tables,
                           int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
                           int window, float scale, float* partial, int nsplit) {
-  attention_decode_kernel<D><<<grid, kWave, 0, s>>>(q, q_stride, heads, kv_heads, positions, tables,
-                                                    table_stride, k_pool, v_pool, page_size,
-                                                    window, scale, partial, nsplit);
+  const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
+  attention_decode_kernel<D><<<grid, kDecodeWaves * kWave, 0, s>>>(q, q_stride, out, heads, kv_heads, positions,
+                                                    tables, table_stride, k_pool, v_pool, page_size,
+                                                    magic, window, scale, partial, nsplit);
+  if (nsplit > 1)
+    attention_merge_kernel<D><<<grid.y * heads, kWave, 0, s>>>(partial, out, nsplit);
 }
 
 template <int D>
@@ -693,18 +964,20 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
   SHK_REQUIRE(q && out && positions && tables && k_pool && v_pool && partial && table_stride > 0,
               "attention_decode: null pointer");
   SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0, "attention_decode: q is not 16-byte aligned");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0,
+              "attention_decode: out must be 8-byte and partial 16-byte aligned");
+  SHK_REQUIRE(static_cast<long long>(table_stride) * page_size * page_size < (1ll << 32),
+              "attention_decode: a block table of %d pages of %d is beyond the kernel's range",
+              table_stride, page_size);
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(kv_heads, num_seqs, nsplit);
 #define CALL(D)                                                                              \
-  launch_decode<D>(grid, s, static_cast<const bf16*>(q), q_stride, heads, kv_heads, positions, \
-                   tables, table_stride, static_cast<const bf16*>(k_pool),                   \
+  launch_decode<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, \
+                   kv_heads, positions, tables, table_stride, static_cast<const bf16*>(k_pool),    \
                    static_cast<const bf16*>(v_pool), page_size, window, scale, partial, nsplit)
   SHK_DISPATCH_D(head_dim, CALL)
 #undef CALL
   SHK_LAUNCH_CHECK("attention_decode");
-  attention_merge_kernel<<<num_seqs * heads, head_dim <= 64 ? 64 : 128, 0, s>>>(
-      partial, static_cast<bf16*>(out), head_dim, nsplit);
-  SHK_LAUNCH_CHECK("attention_merge");
   return 0;
 }
 

@@ -38,6 +38,14 @@ HIPCC_FLAGS = [
 ] + os.environ.get("SHRIKE_HIPCC_EXTRA", "").split()
 
 
+# Flags for single sources.  The attention kernels scale their MFMA accumulators
+# between the matrix instructions; in accumulation registers every such step
+# would cost a copy out and a copy back.
+FILE_FLAGS = {
+    "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def sources() -> list[Path]:
     return sorted(CSRC.glob("*.hip"))
 
@@ -48,6 +56,7 @@ def source_hash() -> str:
         h.update(path.name.encode())
         h.update(path.read_bytes())
     h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
 
@@ -115,7 +124,8 @@ def build(force: bool = True, verbose: bool = True) -> Path:
 
     def compile_one(src: Path) -> Path:
         obj = obj_dir / (src.stem + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+        cmd = [hipcc, *HIPCC_FLAGS, *FILE_FLAGS.get(src.name, []), "-I", str(CSRC), "-c", str(src),
+               "-o", str(obj)]
         proc = subprocess.run(cmd, capture_output=True, text=True)
         if proc.returncode != 0:
             raise RuntimeError(f"hipcc failed on {src.name}:\n{proc.stderr[-4000:]}")

@@ -27,31 +27,63 @@ __global__ void __launch_bounds__(kRopeThreads)
   const int pos = positions[t];
   const int half = rot_dim / 2;
   const int width = (heads + 2 * kv_heads) * head_dim;
-  for (int i = threadIdx.x; i < half; i += kRopeThreads) {
-    // The angle is the float32 product, as the reference forms it; it reaches
-    // thousands of radians, so it is brought into [-pi, pi] in float64 (exact
-    // to 1e-13) before the float32 sine and cosine.
-    const float angle = static_cast<float>(pos) * inv_freq[i];
-    const double a = static_cast<double>(angle);
-    const double turns = rint(a * 0.15915494309189535);
-    const float reduced = static_cast<float>(fma(turns, -6.283185307179586, a));
-    float s, c;
-    sincosf(reduced, &s, &c);
-    cs[i] = c;
-    sn[i] = s;
-  }
-  __syncthreads();
-
   T* row = qkv + static_cast<size_t>(t) * width;
-  // column `col` of this token's projections
-  auto in = [&](int col) -> float {
-    if (splits == 0) return to_float(row[col]);
-    const size_t split_stride = static_cast<size_t>(n) * width;
-    const float* p = parts + static_cast<size_t>(t) * width + col;
-    float v = p[0];
-    for (int z = 1; z < splits; ++z) v += p[z * split_stride];
-    return bias ? v + bias[col] : v;
-  };
+
+  // What this thread moves: a rotated pair, an element behind the rotated part,
+  // or an element of the values.  Its inputs are requested first, so that they
+  // travel while the cosines and sines are tabulated.
+  const int tail = head_dim - rot_dim;  // elements that are not rotated
+  const int n_pairs = (heads + kv_heads) * half;
+  const int n_tail = (heads + kv_heads) * tail;
+  const int n_values = kv_heads * head_dim;
+  const int item = blockIdx.y * kRopeThreads + threadIdx.x;
+  enum { kPairItem, kTailItem, kValueItem, kNone } role = kNone;
+  int h = 0, i = 0, col = 0;
+  if (item < n_pairs) {
+    role = kPairItem;
+    h = item / half, i = item % half;
+    col = h * head_dim + i;
+  } else if (item < n_pairs + n_tail) {
+    role = kTailItem;
+    const int e = item - n_pairs;
+    h = e / tail, i = rot_dim + e % tail;
+    col = h * head_dim + i;
+  } else if (item < n_pairs + n_tail + n_values) {
+    role = kValueItem;
+    i = item - n_pairs - n_tail;  // kv head * head_dim + element
+    col = (heads + kv_heads) * head_dim + i;
+  }
+  // columns `col` and (for a pair) `col + half` of this token's projections; the
+  // parts of a split product are added in order, eight of them in flight
+  float x1 = 0.f, x2 = 0.f;
+  if (role != kNone) {
+    const bool two = role == kPairItem;
+    if (splits == 0) {
+      x1 = to_float(row[col]);
+      if (two) x2 = to_float(row[col + half]);
+    } else {
+      const size_t split_stride = static_cast<size_t>(n) * width;
+      const float* p = parts + static_cast<size_t>(t) * width + col;
+      for (int z0 = 0; z0 < splits; z0 += 8) {
+        float a[8], b[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const bool have = z0 + u < splits;
+          a[u] = have ? p[(z0 + u) * split_stride] : 0.f;
+          b[u] = have && two ? p[(z0 + u) * split_stride + half] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          x1 += a[u];
+          x2 += b[u];
+        }
+      }
+      if (bias) {
+        x1 += bias[col];
+        if (two) x2 += bias[col + half];
+      }
+    }
+  }
 
   int page = -1;
   if (write_kv) {
@@ -64,16 +96,22 @@ __global__ void __launch_bounds__(kRopeThreads)
   // keys [page][kv head][slot][head_dim]; values transposed [page][kv head][head_dim][slot]
   const size_t page_base = static_cast<size_t>(page < 0 ? 0 : page) * kv_heads * page_size * head_dim;
 
-  const int tail = head_dim - rot_dim;  // elements that are not rotated
-  const int n_pairs = (heads + kv_heads) * half;
-  const int n_tail = (heads + kv_heads) * tail;
-  const int n_values = kv_heads * head_dim;
-  const int item = blockIdx.y * kRopeThreads + threadIdx.x;
+  for (int f = threadIdx.x; f < half; f += kRopeThreads) {
+    // The angle is the float32 product, as the reference forms it; it reaches
+    // thousands of radians, so it is brought into [-pi, pi] in float64 (exact
+    // to 1e-13) before the float32 sine and cosine.
+    const float angle = static_cast<float>(pos) * inv_freq[f];
+    const double a = static_cast<double>(angle);
+    const double turns = rint(a * 0.15915494309189535);
+    const float reduced = static_cast<float>(fma(turns, -6.283185307179586, a));
+    float sv, cv;
+    sincosf(reduced, &sv, &cv);
+    cs[f] = cv;
+    sn[f] = sv;
+  }
+  __syncthreads();
 
-  if (item < n_pairs) {
-    const int h = item / half, i = item % half;
-    const int col = h * head_dim + i;
-    const float x1 = in(col), x2 = in(col + half);
+  if (role == kPairItem) {
     const float o1 = x1 * cs[i] - x2 * sn[i], o2 = x2 * cs[i] + x1 * sn[i];
     if (h < heads) {
       row[col] = from_float<T>(o1);
@@ -83,21 +121,15 @@ __global__ void __launch_bounds__(kRopeThreads)
       dst[i] = from_float<T>(o1);
       dst[i + half] = from_float<T>(o2);
     }
-  } else if (item < n_pairs + n_tail) {
-    const int e = item - n_pairs;
-    const int h = e / tail, i = rot_dim + e % tail;
-    const float x = in(h * head_dim + i);
+  } else if (role == kTailItem) {
     if (h < heads) {
-      row[h * head_dim + i] = from_float<T>(x);
+      row[col] = from_float<T>(x1);
     } else if (page >= 0) {
       k_pool[page_base + (static_cast<size_t>(h - heads) * page_size + slot) * head_dim + i] =
-          from_float<T>(x);
+          from_float<T>(x1);
     }
-  } else if (item < n_pairs + n_tail + n_values) {
-    const int e = item - n_pairs - n_tail;  // kv head * head_dim + element
-    if (page >= 0)
-      v_pool[page_base + static_cast<size_t>(e) * page_size + slot] =
-          from_float<T>(in((heads + kv_heads) * head_dim + e));
+  } else if (role == kValueItem) {
+    if (page >= 0) v_pool[page_base + static_cast<size_t>(i) * page_size + slot] = from_float<T>(x1);
   }
 }
 

@@ -121,10 +121,11 @@ def bucket(n: int, floor: int = 1) -> int:
 
 
 def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
-    """Wavefronts per (sequence, key/value head): enough to fill the chip
-    (about 2048 in all), each with at least 128 keys.  Both inputs are rounded
-    up to powers of two first, so a step gives the same result whether it runs
-    kernel by kernel or as a graph captured for its bucket."""
-    want = -(-2048 // (bucket(num_seqs) * kv_heads))
-    most = max(1, bucket(max_ctx, 256) // 128)
+    """Workgroups per (sequence, key/value head) of decode attention: enough to
+    put one on every compute unit (256), each with at least 256 keys for its
+    four wavefronts.  Both inputs are rounded up to powers of two first, so a
+    step gives the same result whether it runs kernel by kernel or as a graph
+    captured for its bucket."""
+    want = -(-256 // (bucket(num_seqs) * kv_heads))
+    most = max(1, bucket(max_ctx, 256) // 256)
     return max(1, min(want, most, 64))
