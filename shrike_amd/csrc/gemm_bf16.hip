@@ -45,7 +45,7 @@ __device__ __forceinline__ Frag load_act(const bf16* __restrict__ a, int lda, in
   return f;
 }
 
-constexpr int kSkinnyBatch = 4;  // k-tiles a wavefront has in flight per buffer
+constexpr int kSkinnyBatch = 2;  // k-tiles a wavefront has in flight per buffer
 
 // One batch of operands: kSkinnyBatch weight tiles and the matching activations.
 // (RB = 2 for the gated variant: the tiles of a gate block and of its up block.)
@@ -53,6 +53,7 @@ template <int NB, int RB>
 struct SkinnyBatch {
   Frag w[kSkinnyBatch][RB];
   Frag x[kSkinnyBatch][NB];
+  uint32_t keep[kSkinnyBatch];  // all ones, or zero where x[u] lies beyond the matrix
 };
 
 __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); }
@@ -81,6 +82,42 @@ __device__ __forceinline__ void skinny_load(SkinnyBatch<NB, RB>& b, const uint4*
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb)
       b.x[u][nb] = load_act(a, lda, n, k, nb * 16 + j, tt * 32 + kg * 8, vec);
+  }
+}
+
+// The same batch without a branch, for 16-byte aligned rows with k % 8 == 0
+// (the usual case): every address is clamped into the matrices and what lies
+// beyond them is zeroed afterwards.  A load under a condition would make the
+// compiler wait, at every use of an operand, for all loads in flight, the next
+// batch's included.  arow[nb]: the lane's activation row (token nb*16 + j,
+// clamped to the last token), at column kg*8 when k >= 32.
+template <int NB, int RB>
+__device__ __forceinline__ void skinny_load_aligned(SkinnyBatch<NB, RB>& b,
+                                                    const uint4* __restrict__ wrow,
+                                                    const bf16* const (&arow)[NB], int k,
+                                                    int ktiles, int t, int step, int kg,
+                                                    int blocks) {
+#pragma unroll
+  for (int u = 0; u < kSkinnyBatch; ++u) {
+    const int tt = t + u * step;
+    const int ttc = tt < ktiles ? tt : ktiles - 1;
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) {
+      // a block beyond the matrix reads block 0 again; its rows are never written
+      const int rbc = rb < blocks ? rb : 0;
+      const uint4* p = wrow + (static_cast<size_t>(rbc) * ktiles + ttc) * kWave;
+      b.w[u][rb].u.x = __builtin_nontemporal_load(&p->x);
+      b.w[u][rb].u.y = __builtin_nontemporal_load(&p->y);
+      b.w[u][rb].u.z = __builtin_nontemporal_load(&p->z);
+      b.w[u][rb].u.w = __builtin_nontemporal_load(&p->w);
+    }
+    const int col = tt * 32 + kg * 8;
+    const bool inside = col < k;  // false for every tile at or beyond ktiles as well
+    b.keep[u] = inside ? ~0u : 0u;  // applied when the operand is used, not while it travels
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      b.x[u][nb].u = *reinterpret_cast<const uint4*>(arow[nb] + (inside ? col : 0));
+    }
   }
 }
 
@@ -123,24 +160,64 @@ __global__ void __launch_bounds__(WAVES* kWave)
     for (int b = 0; b < NB; ++b) acc[rb][b] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // k-tile t belongs to wavefront (t % (WAVES * ksplit)) of the block's ksplit workgroups
-  SkinnyBatch<NB, RB> cur, next;
   const int lanes_k = WAVES * ksplit;  // wavefronts that share the block's k-tiles
   const int kStride = kSkinnyBatch * lanes_k;
   const int t0 = z * WAVES + wave;
-  skinny_load<NB, RB>(cur, wrow, a, lda, n, k, ktiles, t0, lanes_k, j, kg, vec, blocks);
-  for (int t = t0; t < ktiles; t += kStride) {
-    if (t + kStride < ktiles)
-      skinny_load<NB, RB>(next, wrow, a, lda, n, k, ktiles, t + kStride, lanes_k, j, kg, vec,
-                          blocks);
+  auto multiply = [&](const SkinnyBatch<NB, RB>& bt, bool masked) {
 #pragma unroll
     for (int u = 0; u < kSkinnyBatch; ++u)
 #pragma unroll
-      for (int rb = 0; rb < RB; ++rb)
+      for (int b = 0; b < NB; ++b) {
+        Frag x = bt.x[u][b];
+        if (masked) {
+          const uint32_t keep = bt.keep[u];
+          x.u = make_uint4(x.u.x & keep, x.u.y & keep, x.u.z & keep, x.u.w & keep);
+        }
 #pragma unroll
-        for (int b = 0; b < NB; ++b)
-          acc[rb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(cur.w[u][rb].v, cur.x[u][b].v,
-                                                               acc[rb][b], 0, 0, 0);
-    cur = next;
+        for (int rb = 0; rb < RB; ++rb)
+          acc[rb][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bt.w[u][rb].v, x.v, acc[rb][b], 0,
+                                                               0, 0);
+      }
+  };
+  // Two batches of tiles in registers: one is in flight while the other is multiplied.
+  SkinnyBatch<NB, RB> ping, pong;
+  if (vec) {
+    const bf16* arow[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      const int token = nb * 16 + j < n ? nb * 16 + j : n - 1;
+      arow[nb] = a + static_cast<size_t>(token) * lda;
+    }
+    auto load = [&](SkinnyBatch<NB, RB>& bt, int t) {
+      skinny_load_aligned<NB, RB>(bt, wrow, arow, k, ktiles, t, lanes_k, kg, blocks);
+      // the loads go out here, before the other batch's multiplications, not among them
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // every step of the loop issues one batch of loads and multiplies the other
+    int t = t0;
+    load(ping, t);
+    for (; t + 2 * kStride < ktiles; t += 2 * kStride) {
+      load(pong, t + kStride);
+      multiply(ping, true);
+      load(ping, t + 2 * kStride);
+      multiply(pong, true);
+    }
+    if (t + kStride < ktiles) {
+      load(pong, t + kStride);
+      multiply(ping, true);
+      multiply(pong, true);
+    } else {
+      multiply(ping, true);
+    }
+  } else {
+    skinny_load<NB, RB>(ping, wrow, a, lda, n, k, ktiles, t0, lanes_k, j, kg, false, blocks);
+    for (int t = t0; t < ktiles; t += kStride) {
+      if (t + kStride < ktiles)
+        skinny_load<NB, RB>(pong, wrow, a, lda, n, k, ktiles, t + kStride, lanes_k, j, kg, false,
+                            blocks);
+      multiply(ping, false);
+      ping = pong;
+    }
   }
 
 #pragma unroll
