@@ -19,6 +19,9 @@ namespace shk {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+// 16 bytes as the compiler's own vector type: copies of it are loads and stores,
+// where copies of HIP's uint4 struct can end up as memcpy through scratch memory
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 union Frag {
   uint4 u;
@@ -414,12 +417,13 @@ __global__ void __launch_bounds__(WAVES* kWave)
   }
 }
 
-// gemm_big_kernel: for many tokens (prompt portions).  A workgroup of 4
-// wavefronts computes a tile of weight rows x tokens, each wavefront a
-// quadrant of it as WM x WN MFMA tiles.  Per stage of k, the weights' tiles (already in operand layout) and the activations (re-laid on the way)
-// are staged in LDS "fragment-major": the 16 bytes of lane l of a fragment sit
-// at l * 16, so every LDS access is a conflict-free 128-bit access.  Stages are
-// double-buffered: the loads of stage t+1 are in flight while stage t is
+// gemm_big_kernel: for many tokens (prompt portions).  A workgroup of 4 or 8
+// wavefronts computes a tile of weight rows x tokens, each wavefront a part of
+// it as WM x WN MFMA tiles.  Per stage of k, the weights' tiles (already in
+// operand layout) and the activations (re-laid on the way) are staged in LDS
+// "fragment-major": the 16 bytes of lane l of a fragment sit at l * 16, so every
+// LDS access is a conflict-free 128-bit access.  Two LDS buffers alternate, and
+// the loads of the next two stages are in flight (in registers) while a stage is
 // multiplied.
 
 // GM x GN wavefronts per workgroup, each with WM x WN MFMA tiles (16 x 16): the
@@ -427,10 +431,11 @@ __global__ void __launch_bounds__(WAVES* kWave)
 // k) per stage.  The stages live in dynamic LDS, [buffer][fragment][lane].
 template <int GM, int GN, int WM, int WN, int KS, bool GATED>
 __global__ void __launch_bounds__(GM* GN* kWave)
+    __attribute__((amdgpu_waves_per_eu(GM* GN >= 8 || WM * WN <= 16 ? 2 : 1)))
     gemm_big_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                     const uint4* __restrict__ wt, int ktiles, int m,
                     const float* __restrict__ bias, void* __restrict__ out, int ldo, int out_f32,
-                    int accumulate, int vec) {
+                    int accumulate, int vec, int ksplit) {
   constexpr int kWaves = GM * GN;
   constexpr int kWFrags = GM * WM * KS, kAFrags = GN * WN * KS;  // fragments per stage
   constexpr int kFrags = kWFrags + kAFrags;
@@ -442,7 +447,12 @@ __global__ void __launch_bounds__(GM* GN* kWave)
   const int tok0 = blockIdx.y * (16 * GN * WN);
   // blocks of 16 weight rows; a gated weight has two per 16 output rows
   const int mblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
-  const int nstages = (ktiles + KS - 1) / KS;
+  // blockIdx.z: which share of the k stages (ksplit workgroups per tile leave float32
+  // partial sums [ksplit][n][m] that the reading kernel adds up)
+  const int all_stages = (ktiles + KS - 1) / KS;
+  const int per_split = (all_stages + ksplit - 1) / ksplit;
+  const int st_first = blockIdx.z * per_split;
+  const int nstages = st_first + per_split < all_stages ? st_first + per_split : all_stages;
 
   f32x4 acc[WM][WN];
 #pragma unroll
@@ -479,28 +489,112 @@ __global__ void __launch_bounds__(GM* GN* kWave)
       if (wave + kWaves * i < kAFrags) stage(buf, kWFrags + wave + kWaves * i)[lane] = areg[i];
   };
 
-  load_stage(0);
-  store_stage(0);
-  __syncthreads();
-  for (int st = 0; st < nstages; ++st) {
-    const int buf = st & 1;
-    if (st + 1 < nstages) load_stage(st + 1);
+  // every fragment of the stage is requested from LDS before the first multiplication,
+  // so that the later reads travel under the earlier multiplications
+  auto multiply = [&](int buf) {
+    u32x4 af[KS][WN], wf[KS][WM];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      Frag af[WN];
 #pragma unroll
-      for (int jn = 0; jn < WN; ++jn) af[jn].u = stage(buf, kWFrags + (wn * WN + jn) * KS + ks)[lane];
+      for (int jn = 0; jn < WN; ++jn)
+        af[ks][jn] = *reinterpret_cast<const u32x4*>(stage(buf, kWFrags + (wn * WN + jn) * KS + ks) + lane);
 #pragma unroll
-      for (int i = 0; i < WM; ++i) {
-        Frag wf;
-        wf.u = stage(buf, (wm * WM + i) * KS + ks)[lane];
+      for (int i = 0; i < WM; ++i)
+        wf[ks][i] = *reinterpret_cast<const u32x4*>(stage(buf, (wm * WM + i) * KS + ks) + lane);
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int jn = 0; jn < WN; ++jn)
-          acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf.v, af[jn].v, acc[i][jn], 0, 0, 0);
-      }
+          acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, wf[ks][i]), __builtin_bit_cast(bf16x8, af[ks][jn]),
+              acc[i][jn], 0, 0, 0);
+  };
+
+  if (vec && kWFrags % kWaves == 0 && kAFrags % kWaves == 0) {
+    // Aligned rows: every load is unconditional, its address clamped into the
+    // matrices (what an activation row holds past k meets the zeros that pad the
+    // weight tiles), and the loads of two stages are in flight while a stage is
+    // multiplied.
+    const uint4* wsrc[kWPer];
+    const bf16* asrc[kAPer];
+#pragma unroll
+    for (int i = 0; i < kWPer; ++i) {
+      const int rb = (wave + kWaves * i) / KS;
+      const int block = mb0 + rb < mblocks ? mb0 + rb : mblocks - 1;
+      wsrc[i] = wt + static_cast<size_t>(block) * ktiles * kWave + lane;
     }
-    if (st + 1 < nstages) store_stage(buf ^ 1);
+#pragma unroll
+    for (int i = 0; i < kAPer; ++i) {
+      const int rb = (wave + kWaves * i) / KS;
+      const int token = tok0 + rb * 16 + lane % 16;
+      asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (lane / 16) * 8;
+    }
+    // Two named sets of registers, not an array of two: an array indexed by the
+    // loop's step would live in scratch memory.
+    u32x4 even_w[kWPer], even_x[kAPer], odd_w[kWPer], odd_x[kAPer];
+    auto fetch = [&](u32x4 (&hw)[kWPer], u32x4 (&hx)[kAPer], int st) {
+#pragma unroll
+      for (int i = 0; i < kAPer; ++i) {
+        const int col = (st * KS + (wave + kWaves * i) % KS) * 32;  // + (lane / 16) * 8 in asrc
+        hx[i] = *reinterpret_cast<const u32x4*>(asrc[i] + (col + (lane / 16) * 8 < k ? col : 0));
+      }
+#pragma unroll
+      for (int i = 0; i < kWPer; ++i) {
+        const int kt = st * KS + (wave + kWaves * i) % KS;
+        hw[i] = *reinterpret_cast<const u32x4*>(wsrc[i] + static_cast<size_t>(kt < ktiles ? kt : 0) * kWave);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // the loads go out before the multiplications
+    };
+    auto put = [&](const u32x4 (&hw)[kWPer], const u32x4 (&hx)[kAPer], int st, int buf) {
+#pragma unroll
+      for (int i = 0; i < kWPer; ++i)
+        *reinterpret_cast<u32x4*>(stage(buf, wave + kWaves * i) + lane) = hw[i];
+#pragma unroll
+      for (int i = 0; i < kAPer; ++i) {
+        // a k-tile past the last one (the stage is not full) must contribute nothing
+        const uint32_t keep = st * KS + (wave + kWaves * i) % KS < ktiles ? ~0u : 0u;
+        *reinterpret_cast<u32x4*>(stage(buf, kWFrags + wave + kWaves * i) + lane) = hx[i] & keep;
+      }
+    };
+    // stage st is multiplied from LDS buffer st % 2 while the loads of stages
+    // st + 1 (issued a step ago) and st + 2 (issued now) are in flight
+    fetch(even_w, even_x, st_first);
+    fetch(odd_w, odd_x, st_first + 1);
+    put(even_w, even_x, st_first, 0);
     __syncthreads();
+    // The loop's body has no branch: with one, the compiler moves loads behind it,
+    // next to their use, and nothing is in flight any more.
+    int st = st_first;
+    for (; st + 2 < nstages; st += 2) {
+      fetch(even_w, even_x, st + 2);
+      multiply(0);
+      put(odd_w, odd_x, st + 1, 1);
+      __syncthreads();
+      fetch(odd_w, odd_x, st + 3);
+      multiply(1);
+      put(even_w, even_x, st + 2, 0);
+      __syncthreads();
+    }
+    if (st < nstages) multiply(0);
+    if (st + 1 < nstages) {
+      put(odd_w, odd_x, st + 1, 1);
+      __syncthreads();
+      multiply(1);
+    }
+  } else {
+    load_stage(st_first);
+    store_stage(0);
+    __syncthreads();
+    for (int st = st_first; st < nstages; ++st) {
+      const int buf = (st - st_first) & 1;
+      if (st + 1 < nstages) load_stage(st + 1);
+      multiply(buf);
+      if (st + 1 < nstages) store_stage(buf ^ 1);
+      __syncthreads();
+    }
   }
 
   // lane (j, kg) of tile (i, jn): token tok0 + (wn*WN + jn)*16 + j,
@@ -521,7 +615,7 @@ __global__ void __launch_bounds__(GM* GN* kWave)
         v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r] : acc[i][jn][r];
         if (bias && row0 + r < m) v[r] += bias[row0 + r];
       }
-      const size_t idx = static_cast<size_t>(token) * ldo + row0;
+      const size_t idx = (static_cast<size_t>(blockIdx.z) * n + token) * ldo + row0;
       if (out_f32) {
         float* o = static_cast<float*>(out) + idx;
 #pragma unroll
@@ -602,9 +696,43 @@ extern "C" int shk_interleave_gate_up(const void* gate_t, const void* up_t, int 
 // Workgroups per block of 16 weight rows that a product with at most 64 rows
 // should be split into along k so that the chip is full (about 8192 wavefronts
 // with 4 k-tiles or more each): 1 for matrices with many row blocks.
+template <int GM, int GN, int WM, int WN, int KS>
+static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, const uint4* wp, int kt,
+                       int m, const float* bias, void* out, int ldo, int of, int accumulate, int vec,
+                       int gated, int wblocks, int ksplit) {
+  constexpr int lds = 2 * (GM * WM + GN * WN) * KS * kWave * 16;
+  dim3 grid((wblocks + GM * WM - 1) / (GM * WM), (n + 16 * GN * WN - 1) / (16 * GN * WN), ksplit);
+  if (gated) {
+    auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, true>;
+    if (lds > 65536)
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate,
+                                              vec, ksplit);
+  } else {
+    auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, false>;
+    if (lds > 65536)
+      hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+    kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate,
+                                              vec, ksplit);
+  }
+}
+
 extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   const int mblocks = (m + 15) / 16, ktiles = (k + 31) / 32;
-  if (n > 64 || mblocks >= 512) return 1;
+  if (n > 64) {
+    // many tokens: tiles of 128 x 128; split k when they leave half the chip idle,
+    // each share keeping at least 8 stages of 64
+    const long long tiles = static_cast<long long>((mblocks + 7) / 8) * ((n + 127) / 128);
+    if (tiles >= 128) return 1;
+    int split = static_cast<int>(256 / tiles);
+    const int most = ktiles / 16;
+    if (split > most) split = most;
+    if (split > 16) split = 16;
+    return split > 1 ? split : 1;
+  }
+  if (mblocks >= 512) return 1;
   // up to 16 tokens: workgroups of 4 wavefronts share a block's k-tiles; more tokens:
   // workgroups of 4 blocks walk k in stages of 4 tiles
   int split = n <= 16 ? 8192 / (mblocks * 4) : 1024 / ((mblocks + 3) / 4);
@@ -620,9 +748,8 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
                                           void* stream) {
   SHK_REQUIRE(!gated || (!accumulate && !bias), "gemm_bf16: a gated product takes no bias and does not accumulate");
   SHK_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_bf16: ksplit %d is outside 1..64", ksplit);
-  SHK_REQUIRE(ksplit == 1 || (n <= 64 && !gated && !accumulate && !bias && out_dtype == kF32 && ldo == m),
-              "gemm_bf16: a product split along k has at most 64 rows and writes plain float32 "
-              "partial sums [ksplit][n][m]");
+  SHK_REQUIRE(ksplit == 1 || (!gated && !accumulate && !bias && out_dtype == kF32 && ldo == m),
+              "gemm_bf16: a product split along k writes plain float32 partial sums [ksplit][n][m]");
   SHK_REQUIRE(out_dtype == kF32 || out_dtype == kBF16, "gemm_bf16: unknown out_dtype %d",
               out_dtype);
   SHK_REQUIRE(n >= 0 && m > 0 && k > 0, "gemm_bf16: bad sizes n=%d m=%d k=%d", n, m, k);
@@ -639,31 +766,20 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   if (n > 64) {
     SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
     const int wblocks = (gated ? 2 : 1) * mb;  // blocks of 16 weight rows
-#define SHK_BIG(GM, GN, WM, WN, KS)                                                            \
-  do {                                                                                         \
-    constexpr int lds = 2 * (GM * WM + GN * WN) * KS * kWave * 16;                             \
-    dim3 grid((wblocks + GM * WM - 1) / (GM * WM), (n + 16 * GN * WN - 1) / (16 * GN * WN));   \
-    SHK_REQUIRE(grid.y <= 65535, "gemm_bf16: too many rows (%d)", n);                          \
-    if (gated) {                                                                               \
-      auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, true>;                                 \
-      if (lds > 65536)                                                                         \
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                             \
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);                  \
-      kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,  \
-                                                accumulate, vec);                              \
-    } else {                                                                                   \
-      auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, false>;                                \
-      if (lds > 65536)                                                                         \
-        hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),                             \
-                            hipFuncAttributeMaxDynamicSharedMemorySize, lds);                  \
-      kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of,  \
-                                                accumulate, vec);                              \
-    }                                                                                          \
-  } while (0)
-    // 128 x 128 per workgroup, 64 of k per stage (128 x 256 with eight wavefronts
-    // measured slower: the staging, not the arithmetic, bounds this kernel)
-    SHK_BIG(2, 2, 4, 4, 2);
-#undef SHK_BIG
+    // Tile of the workgroup: the largest of 256 x 256, 256 x 128 and 128 x 128
+    // (weight rows x tokens) that still gives every compute unit a workgroup.
+    auto tiles = [&](int rows, int tokens) {
+      return static_cast<long long>((wblocks * 16 + rows - 1) / rows) * ((n + tokens - 1) / tokens);
+    };
+    if (ksplit == 1 && tiles(256, 256) >= 256)
+      launch_big<4, 2, 4, 8, 1>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+                                gated, wblocks, ksplit);
+    else if (ksplit == 1 && tiles(256, 128) >= 200)
+      launch_big<4, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+                                gated, wblocks, ksplit);
+    else
+      launch_big<2, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+                                gated, wblocks, ksplit);
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }

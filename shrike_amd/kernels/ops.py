@@ -168,7 +168,8 @@ def gemm_splits(n: int, m: int, k: int) -> int:
 def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, gated=False,
                       splits: int = 1) -> None:
     """out (+)= a @ w.T + bias with wt = retile_weight(w): up to 64 rows of a
-    stream the weights once; more rows run the LDS-staged MFMA kernel.
+    stream the weights once; more rows run the LDS-staged MFMA kernel (tiles of
+    128 x 128 to 256 x 256, chosen by how many the product has).
     splits > 1: out is float32 [splits, n, m] and receives partial sums."""
     _rows(a, "gemm a")
     n = a.shape[0]
