@@ -668,19 +668,25 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
 }
 
 // ------------------------------------------------- prefill, keys shared in LDS
-// A workgroup of 4 wavefronts serves every query head of one key/value head for
-// a run of 16-query tiles of one sequence: the chunk of 32 keys is fetched once,
-// staged in LDS in operand layout and read by all of them, instead of once per
-// (head, tile).  A wavefront owns two "units" (query head, query tile); unit
-// u < tiles * group is tile u / group, head u % group of the key/value head.
+// A workgroup of 8 wavefronts serves every query head of one key/value head for
+// a run of 16-query tiles of one sequence.  The chunk of 32 keys is fetched once
+// and staged in LDS in operand layout; a wavefront owns two "units" (query head,
+// query tile) and multiplies every fragment it reads from LDS with both.  The
+// softmax arithmetic, not the matrix unit, bounds a wavefront, and the workgroup
+// with the last queries sets the kernel's time, hence many wavefronts with
+// little each (four with four units measured 1.5 times slower).  Unit u < tiles *
+// group is tile u / group, head u % group of the key/value head.  The products
+// are formed transposed as in the decode kernel (S^T = K Q^T, O^T += V^T P^T):
+// a lane owns one query, and P needs no trip through LDS.
 // grid (workgroup tiles, kv_heads); wg_seq / wg_q0 as tile_seq / tile_q0 above,
 // in steps of 16 * tiles queries.
 
 constexpr int kUnitsPerWave = 2;
-constexpr int kSharedWaves = 4;
+constexpr int kSharedWaves = 8;
 
 template <int D>
-__global__ void __launch_bounds__(kSharedWaves* kWave) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(kSharedWaves* kWave)
+    __attribute__((amdgpu_waves_per_eu(kUnitsPerWave <= 2 || kSharedWaves > 4 ? 2 : 1)))
     attention_prefill_shared_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                                     int heads, int kv_heads, int tiles,
                                     const int32_t* __restrict__ cu_q,
@@ -689,14 +695,17 @@ __global__ void __launch_bounds__(kSharedWaves* kWave) __attribute__((amdgpu_wav
                                     const int32_t* __restrict__ wg_q0,
                                     const int32_t* __restrict__ tables, int table_stride,
                                     const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
-                                    int page_size, int window, float scale) {
+                                    int page_size, uint32_t page_magic, int window, float scale) {
+  constexpr int U = kUnitsPerWave;
   constexpr int kKFrags = 2 * (D / 32), kVFrags = D / 16, kFrags = kKFrags + kVFrags;
-  constexpr int kPerThread = kFrags / kSharedWaves;  // fragments each wavefront stages
-  __shared__ uint4 kv[2][kFrags][kWave];
-  __shared__ __attribute__((aligned(16))) uint16_t p_all[kSharedWaves][16 * kPStride];
+  // fragments each wavefront stages; where they do not divide, some are staged twice
+  constexpr int kPer = (kFrags + kSharedWaves - 1) / kSharedWaves;
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  __shared__ u32x4 kv[2][kFrags][kWave];
 
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
-  const int j = lane % 16, kg = lane / 16;
+  const int j = lane % 16, g = lane / 16;
+  const PageDiv pd{page_size, page_magic};
   // workgroups are listed in token order; the last ones read the most keys, so they start first
   const int wg = gridDim.x - 1 - blockIdx.x;
   const int seq = wg_seq[wg], q0 = wg_q0[wg], kvh = blockIdx.y;
@@ -704,176 +713,213 @@ __global__ void __launch_bounds__(kSharedWaves* kWave) __attribute__((amdgpu_wav
   const int tok0 = cu_q[seq], q_len = cu_q[seq + 1] - tok0;
   const int start = ctx_lens[seq] - q_len;  // position of the portion's first token
   const int q_end = (q0 + 16 * tiles < q_len) ? q0 + 16 * tiles : q_len;
-  const int ps = page_size;
-  const size_t head_elems = static_cast<size_t>(ps) * D;
+  const size_t head_elems = static_cast<size_t>(page_size) * D;
   const int32_t* table = tables + static_cast<size_t>(seq) * table_stride;
-  uint16_t* p_lds = p_all[wave];
 
   // bounds over the whole workgroup: what has to be staged
   const int pos_min = start + q0, pos_max = start + q_end - 1;
   const int lo_min = (window > 0 && pos_min - window + 1 > 0) ? pos_min - window + 1 : 0;
   const int key_begin = lo_min & ~31;
+  const int nchunks = (pos_max - key_begin) / 32 + 1;
 
-  // this wavefront's units
-  AFrag qf[kUnitsPerWave][D / 32];
-  int row_pos[kUnitsPerWave][4], row_lo[kUnitsPerWave][4];
-  float m[kUnitsPerWave][4], l[kUnitsPerWave][4];
-  f32x4 o[kUnitsPerWave][D / 16];
-  int unit_head[kUnitsPerWave], unit_q0[kUnitsPerWave], unit_rows[kUnitsPerWave];
+  // this wavefront's units; a lane owns query j of each
+  AFrag qf[U][D / 32];
+  int q_pos[U], q_lo[U];  // last and first key this lane's query reads (-1: no query)
+  float m[U], l[U];       // base-2 logarithms; l is the lane's share of the sum until the end
+  f32x4 o[U][D / 16];     // element db*16 + 4*g + r of the lane's query
+  int unit_head[U], unit_q0[U], unit_rows[U];
+  const float scale2 = scale * 1.4426950408889634f;
 #pragma unroll
-  for (int u = 0; u < kUnitsPerWave; ++u) {
-    const int unit = wave * kUnitsPerWave + u;
+  for (int u = 0; u < U; ++u) {
+    const int unit = wave * U + u;
     const bool valid = unit < tiles * group && q0 + (unit / group) * 16 < q_len;
     unit_head[u] = kvh * group + unit % group;
     unit_q0[u] = q0 + (unit / group) * 16;
     unit_rows[u] = !valid ? 0 : (q_len - unit_q0[u] < 16 ? q_len - unit_q0[u] : 16);
-    const bf16* qrow = q + static_cast<size_t>(tok0 + unit_q0[u] + j) * q_stride +
-                       static_cast<size_t>(unit_head[u]) * D + kg * 8;
+    const int qrow_i = j < unit_rows[u] ? j : 0;  // an address inside the portion for every lane
+    const bf16* qrow = q + static_cast<size_t>(tok0 + (valid ? unit_q0[u] : 0) + qrow_i) * q_stride +
+                       static_cast<size_t>(unit_head[u]) * D + g * 8;
 #pragma unroll
     for (int ds = 0; ds < D / 32; ++ds) {
       qf[u][ds].u = make_uint4(0, 0, 0, 0);
       if (j < unit_rows[u]) qf[u][ds].u = *reinterpret_cast<const uint4*>(qrow + ds * 32);
     }
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int qi = kg * 4 + r;
-      row_pos[u][r] = (qi < unit_rows[u]) ? start + unit_q0[u] + qi : -1;
-      row_lo[u][r] = (window > 0 && row_pos[u][r] - window + 1 > 0) ? row_pos[u][r] - window + 1 : 0;
-      m[u][r] = -INFINITY;
-      l[u][r] = 0.f;
-    }
+    q_pos[u] = j < unit_rows[u] ? start + unit_q0[u] + j : -1;
+    q_lo[u] = (window > 0 && q_pos[u] - window + 1 > 0) ? q_pos[u] - window + 1 : 0;
+    m[u] = -INFINITY;
+    l[u] = 0.f;
 #pragma unroll
     for (int db = 0; db < D / 16; ++db) o[u][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // Staging: wavefront w fetches fragments w, w + 4, ...  Fragment f < kKFrags is
-  // K tile f / (D/32), head_dim slice f % (D/32); the others are V blocks of 16 elements.
-  uint4 regs[kPerThread];
-  auto fetch = [&](int kb) {
+  // ---- staging.  Wavefront w fetches fragments w, w + 4, ...  Fragment f < kKFrags
+  // is K tile f / (D/32), head_dim slice f % (D/32); row i of K tile t is key
+  // 8*(i/4) + 4*t + i%4 of the chunk, so that lane (j, g) of a score tile ends up
+  // with the eight keys 8*g .. 8*g + 7.  The others are V^T blocks of 16 elements.
+  // Every load is unconditional (addresses clamped into pages the sequence holds).
+  const bool second_k = j >= 8, second_v = g >= 2;
+  int lane_off[kPer];
+  bool is_k[kPer];
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) {
-      const int f = wave + kSharedWaves * i;
-      regs[i] = make_uint4(0, 0, 0, 0);
-      if (f < kKFrags) {
-        const int tt = f / (D / 32), ds = f % (D / 32);
-        const int key0 = kb + tt * 16;
-        if (key0 <= pos_max && key0 + 15 >= lo_min) {
-          const int page = table[key0 / ps];
-          regs[i] = *reinterpret_cast<const uint4*>(
-              k_pool + (static_cast<size_t>(page) * kv_heads + kvh) * head_elems +
-              static_cast<size_t>(key0 % ps + j) * D + ds * 32 + kg * 8);
-        }
-      } else {
-        const int db = f - kKFrags;
-        const int g0 = kb + kg * 8;
-        if (g0 <= pos_max && g0 + 7 >= lo_min) {
-          const int page = table[g0 / ps];
-          uint4 v = *reinterpret_cast<const uint4*>(
-              v_pool + (static_cast<size_t>(page) * kv_heads + kvh) * head_elems +
-              static_cast<size_t>(db * 16 + j) * ps + g0 % ps);
-          if (g0 < lo_min || g0 + 7 > pos_max) {
-            // keys outside [lo_min, pos_max] carry weight 0 but may hold anything
-            uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const bool a = g0 + 2 * e >= lo_min && g0 + 2 * e <= pos_max;
-              const bool b = g0 + 2 * e + 1 >= lo_min && g0 + 2 * e + 1 <= pos_max;
-              w[e] &= (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
-            }
-            v = make_uint4(w[0], w[1], w[2], w[3]);
-          }
-          regs[i] = v;
-        }
-      }
+  for (int i = 0; i < kPer; ++i) {
+    const int f = (wave + kSharedWaves * i) % kFrags;
+    is_k[i] = f < kKFrags;
+    if (is_k[i]) {
+      const int t = f / (D / 32), ds = f % (D / 32);
+      lane_off[i] = (8 * ((j / 4) % 2) + 4 * t + j % 4) * D + ds * 32 + g * 8;
+    } else {
+      const int db = f - kKFrags;
+      lane_off[i] = (db * 16 + j) * page_size + 8 * (g % 2);
     }
-  };
-  auto stash = [&](int buf) {
+  }
+  auto fetch = [&](u32x4 (&held)[kPer], int chunk) {
+    const int kb = key_begin + 32 * (chunk < nchunks ? chunk : nchunks - 1);
+    int ka = kb < lo_min ? lo_min : kb, kc = kb + 16 < lo_min ? lo_min : kb + 16;
+    ka = ka > pos_max ? pos_max : ka;
+    kc = kc > pos_max ? pos_max : kc;
+    const int page_a = table[__builtin_amdgcn_readfirstlane(pd.div(ka))];
+    const int page_c = table[__builtin_amdgcn_readfirstlane(pd.div(kc))];
+    const size_t head_a = (static_cast<size_t>(page_a) * kv_heads + kvh) * head_elems;
+    const size_t head_c = (static_cast<size_t>(page_c) * kv_heads + kvh) * head_elems;
+    const int slot_a = pd.mod(kb), slot_c = pd.mod(kb + 16);
+    const bf16* krow = k_pool + (second_k ? head_c + static_cast<size_t>(slot_c) * D
+                                          : head_a + static_cast<size_t>(slot_a) * D);
+    const bf16* vcol = v_pool + (second_v ? head_c + slot_c : head_a + slot_a);
 #pragma unroll
-    for (int i = 0; i < kPerThread; ++i) kv[buf][wave + kSharedWaves * i][lane] = regs[i];
+    for (int i = 0; i < kPer; ++i)
+      held[i] = *reinterpret_cast<const u32x4*>((is_k[i] ? krow : vcol) + lane_off[i]);
+    __builtin_amdgcn_sched_barrier(0);  // the loads go out before the multiplications
+  };
+  auto put = [&](const u32x4 (&held)[kPer], int chunk, int buf) {
+    const int kb = key_begin + 32 * chunk;
+    const int g0 = kb + g * 8;  // a V fragment's lane holds keys g0 .. g0 + 7
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      u32x4 x = held[i];
+      if (!is_k[i]) {
+        // keys outside [lo_min, pos_max] carry weight 0, but their slots may hold anything
+        u32x4 keep;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const bool a = g0 + 2 * e >= lo_min && g0 + 2 * e <= pos_max;
+          const bool b = g0 + 2 * e + 1 >= lo_min && g0 + 2 * e + 1 <= pos_max;
+          keep[e] = (a ? 0x0000ffffu : 0u) | (b ? 0xffff0000u : 0u);
+        }
+        x &= keep;
+      }
+      kv[buf][(wave + kSharedWaves * i) % kFrags][lane] = x;
+    }
   };
 
-  fetch(key_begin);
-  stash(0);
-  __syncthreads();
-  int buf = 0;
-  for (int kb = key_begin; kb <= pos_max; kb += 32) {
-    const bool more = kb + 32 <= pos_max;
-    if (more) fetch(kb + 32);
+  // ---- one chunk for this wavefront's units, from LDS buffer `buf`
+  // chunks at or before `last_plain` lie wholly inside what every query of the
+  // workgroup reads (none without a window's lower bound to check)
+  const int last_plain = window > 0 ? -1 : (pos_min + 1 - key_begin) / 32 - 1;
+  auto attend = [&](int buf, int chunk) {
+    const int kb = key_begin + 32 * chunk;
+    const int g0 = kb + g * 8;
+    const bool edge = chunk > last_plain;
+    u32x4 kf[2][D / 32];
 #pragma unroll
-    for (int u = 0; u < kUnitsPerWave; ++u) {
-      // ---- S = Q K^T
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int ds = 0; ds < D / 32; ++ds) kf[t][ds] = kv[buf][t * (D / 32) + ds][lane];
+    AFrag pf[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
       f32x4 s[2];
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt) {
-        s[tt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int t = 0; t < 2; ++t) {
+        s[t] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ds = 0; ds < D / 32; ++ds) {
-          AFrag kf;
-          kf.u = kv[buf][tt * (D / 32) + ds][lane];
-          s[tt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[u][ds].v, kf.v, s[tt], 0, 0, 0);
-        }
+        for (int ds = 0; ds < D / 32; ++ds)
+          s[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, kf[t][ds]),
+                                                         qf[u][ds].v, s[t], 0, 0, 0);
       }
-      // ---- mask, running maximum and sum
-      float p[2][4];
+      // this lane's keys are g0 + e, e = 4*t + r
+      float sc[8];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float sc[2];
+      for (int e = 0; e < 8; ++e) sc[e] = s[e / 4][e % 4] * scale2;
+      if (edge) {  // wave-uniform: some query of the workgroup does not read the whole chunk
 #pragma unroll
-        for (int tt = 0; tt < 2; ++tt) {
-          const int key = kb + tt * 16 + j;
-          const bool keep = key <= row_pos[u][r] && key >= row_lo[u][r];
-          sc[tt] = keep ? s[tt][r] * scale : -INFINITY;
-        }
-        const float mx = row16_max(fmaxf(sc[0], sc[1]));
-        const float m_new = fmaxf(m[u][r], mx);
-        const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __expf(m[u][r] - m_safe);
-        p[0][r] = __expf(sc[0] - m_safe);
-        p[1][r] = __expf(sc[1] - m_safe);
-        const float sum = row16_sum(p[0][r] + p[1][r]);
-        l[u][r] = l[u][r] * alpha + sum;
-        m[u][r] = m_new;
-#pragma unroll
-        for (int db = 0; db < D / 16; ++db) o[u][db][r] *= alpha;
+        for (int e = 0; e < 8; ++e)
+          if (g0 + e > q_pos[u] || g0 + e < q_lo[u]) sc[e] = -INFINITY;
       }
-      // ---- P through this wavefront's LDS patch into A-operand layout.  Only this
-      // wavefront touches the patch; the fences order its own writes and reads.
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      __builtin_amdgcn_wave_barrier();
+      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
+                       fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      const float m_new = fmaxf(m[u], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = __builtin_amdgcn_exp2f(m[u] - m_safe);
+      float pr[8];
 #pragma unroll
-      for (int tt = 0; tt < 2; ++tt)
+      for (int e = 0; e < 8; ++e) pr[e] = __builtin_amdgcn_exp2f(sc[e] - m_safe);
+      l[u] = l[u] * alpha +
+             (((pr[0] + pr[1]) + (pr[2] + pr[3])) + ((pr[4] + pr[5]) + (pr[6] + pr[7])));
+      m[u] = m_new;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some query's maximum rose
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          p_lds[(kg * 4 + r) * kPStride + tt * 16 + j] = bf16_bits(p[tt][r]);
-      __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      AFrag pf;
-      pf.u = *reinterpret_cast<const uint4*>(p_lds + j * kPStride + kg * 8);
-      // ---- O += P V
-#pragma unroll
-      for (int db = 0; db < D / 16; ++db) {
-        AFrag vf;
-        vf.u = kv[buf][kKFrags + db][lane];
-        o[u][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf.v, vf.v, o[u][db], 0, 0, 0);
+        for (int db = 0; db < D / 16; ++db) o[u][db] *= alpha;
       }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) pf[u].v[e] = static_cast<__bf16>(pr[e]);
     }
-    if (more) stash(buf ^ 1);
+#pragma unroll
+    for (int db = 0; db < D / 16; ++db) {
+      const u32x4 vf = kv[buf][kKFrags + db][lane];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        o[u][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, vf), pf[u].v,
+                                                           o[u][db], 0, 0, 0);
+    }
+  };
+
+  // Chunk c is multiplied from LDS buffer c % 2 while the loads of chunks c + 1 and
+  // c + 2 are in flight.  The loop's body has no branch, so the loads stay where
+  // they are written.
+  u32x4 even[kPer], odd[kPer];
+  fetch(even, 0);
+  fetch(odd, 1);
+  put(even, 0, 0);
+  __syncthreads();
+  int c = 0;
+  for (; c + 2 < nchunks; c += 2) {
+    fetch(even, c + 2);
+    attend(0, c);
+    put(odd, c + 1, 1);
     __syncthreads();
-    buf ^= 1;
+    fetch(odd, c + 3);
+    attend(1, c + 1);
+    put(even, c + 2, 0);
+    __syncthreads();
+  }
+  attend(0, c);
+  if (c + 1 < nchunks) {
+    put(odd, c + 1, 1);
+    __syncthreads();
+    attend(1, c + 1);
   }
 
 #pragma unroll
-  for (int u = 0; u < kUnitsPerWave; ++u)
+  for (int u = 0; u < U; ++u) {
+    float total = l[u];
+    total += __shfl_xor(total, 16, kWave);
+    total += __shfl_xor(total, 32, kWave);
+    if (j >= unit_rows[u]) continue;
+    const float inv = 1.f / total;
+    bf16* dst = out + static_cast<size_t>(tok0 + unit_q0[u] + j) * heads * D +
+                static_cast<size_t>(unit_head[u]) * D + 4 * g;
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int qi = kg * 4 + r;
-      if (qi >= unit_rows[u]) continue;
-      bf16* dst = out + static_cast<size_t>(tok0 + unit_q0[u] + qi) * heads * D +
-                  static_cast<size_t>(unit_head[u]) * D;
-      const float inv = 1.f / l[u][r];
-#pragma unroll
-      for (int db = 0; db < D / 16; ++db) dst[db * 16 + j] = from_float<bf16>(o[u][db][r] * inv);
+    for (int db = 0; db < D / 16; ++db) {
+      uint2 packed;
+      packed.x = bf16_bits(o[u][db][0] * inv) |
+                 (static_cast<uint32_t>(bf16_bits(o[u][db][1] * inv)) << 16);
+      packed.y = bf16_bits(o[u][db][2] * inv) |
+                 (static_cast<uint32_t>(bf16_bits(o[u][db][3] * inv)) << 16);
+      *reinterpret_cast<uint2*>(dst + db * 16) = packed;
     }
+  }
 }
 
 template <int D>
@@ -908,9 +954,10 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
                                   const int32_t* wg_q0, const int32_t* tables, int table_stride,
                                   const bf16* k_pool, const bf16* v_pool, int page_size, int window,
                                   float scale) {
+  const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
   attention_prefill_shared_kernel<D><<<grid, kSharedWaves * kWave, 0, s>>>(
       q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables, table_stride,
-      k_pool, v_pool, page_size, window, scale);
+      k_pool, v_pool, page_size, magic, window, scale);
 }
 
 }  // namespace shk
@@ -1007,8 +1054,11 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
   SHK_REQUIRE(q && out && cu_q && ctx_lens && wg_seq && wg_q0 && tables && k_pool && v_pool &&
                   table_stride > 0,
               "attention_prefill_shared: null pointer");
-  SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0,
-              "attention_prefill_shared: q is not 16-byte aligned");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(q) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 8 == 0,
+              "attention_prefill_shared: q must be 16-byte and out 8-byte aligned");
+  SHK_REQUIRE(static_cast<long long>(table_stride) * page_size * page_size < (1ll << 32),
+              "attention_prefill_shared: a block table of %d pages of %d is beyond the kernel's range",
+              table_stride, page_size);
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid(num_wgs, kv_heads);
 #define CALL(D)                                                                                \

@@ -593,15 +593,15 @@ def test_rope_kv_store_adds_up_a_split_product(ops):
 @pytest.mark.parametrize(
     "heads, kv_heads, head_dim, page_size, window",
     [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 128, 16, None),
-     (16, 2, 64, 16, 100), (3, 1, 128, 48, None)],
+     (16, 2, 64, 16, 100), (3, 1, 128, 48, None), (16, 1, 32, 16, None), (12, 1, 64, 32, 50)],
 )
 def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window):
     """The prefill kernel that shares each chunk of keys among the query heads of a
-    key/value head: 1 to 8 heads per group, portions of 2 to 200 tokens."""
+    key/value head: 1 to 16 heads per group, portions of 2 to 200 tokens."""
     torch.manual_seed(20)
     dtype = torch.bfloat16
     tiles = ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim)
-    assert tiles == 8 // (heads // kv_heads)
+    assert tiles == 16 // (heads // kv_heads)
     seq_lens = [2, 200, 16, 17, 90, 33, 130]
     starts = [0, 60, 5, 100, 0, 31, 7]
     ctx = [s + l for s, l in zip(starts, seq_lens)]
@@ -629,5 +629,5 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
 
 
 def test_attention_prefill_shared_refuses_wide_groups(ops):
-    assert ops.attention_prefill_shared_tiles(32, 2, 64) == 0  # 16 heads per group: the per-tile kernel serves it
+    assert ops.attention_prefill_shared_tiles(34, 2, 64) == 0  # 17 heads per group: the per-tile kernel serves it
     assert ops.attention_prefill_shared_tiles(8, 2, 256) == 0
