@@ -102,7 +102,7 @@ class ModelRunner:
         self._pinned_free = None  # event: the last copy out of the pinned buffer is done
         # Graphs replay fixed kernel arguments: a mixer that reads host-side
         # metadata (state kept outside the kernels' view) cannot be captured.
-        self.use_graphs = bool(graphs) and not cache.state_groups
+        self.use_graphs = bool(graphs) and not cache.state_groups and model.graph_safe()
         self._graphs: dict[tuple, _DecodeGraph] = {}
         self.graph_replays = 0
 

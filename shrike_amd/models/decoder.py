@@ -36,6 +36,10 @@ class DecoderModel:
         )
         return out
 
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be recorded into a HIP graph."""
+        return all(block.graph_safe for block in self.blocks)
+
     def cache_specs(self) -> list:
         """Cache need of every schedule position (None for a position that
         reads another position's cache or whose mixer keeps nothing)."""

@@ -77,6 +77,11 @@ class HiddenState:
 class Part:
     """Common face of every part."""
 
+    # False for a part whose forward cannot be recorded into a HIP graph (it reads
+    # device data on the host, or launches work whose shape depends on the data);
+    # a model with such a part runs every step kernel by kernel.
+    graph_safe = True
+
     def __init__(self, spec, width: int, name: str):
         self.spec = spec
         self.width = width

@@ -24,6 +24,10 @@ class PreNormResidualBlock(Block):
         for part in self.parts:
             part.check(runtime)
 
+    @property
+    def graph_safe(self):
+        return all(part.graph_safe for part in self.parts)
+
     def load(self, tensors, runtime):
         for part in self.parts:
             part.load(tensors, runtime)

@@ -293,3 +293,158 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
     cache.free(sa)
     cache.free(sb)
     assert plain.rel_err(step_whole(runner, cache, b), wb) <= 1e-5
+
+
+# ------------------------------------- a toy feed-forward that routes its tokens
+
+
+@dataclass(frozen=True)
+class Top1Spec:
+    """y = p_e(x) * W2_e relu(W1_e x), e the expert with the largest router logit,
+    p the softmax of the router logits."""
+
+    kind: ClassVar[str] = "toy_top1"
+    experts: int
+    inner: int
+
+
+def define_toy_routed_ffn():
+    from shrike_amd.parts import FeedForward, ParamSpec, register_ffn
+
+    class Top1Experts(FeedForward):
+        graph_safe = False  # the rows of an expert are gathered on the host's say-so
+
+        def params(self):
+            e, i, w = self.spec.experts, self.spec.inner, self.width
+            out = [ParamSpec(f"{self.name}.router.weight", (e, w), keep_float32=True)]
+            for x in range(e):
+                out += [ParamSpec(f"{self.name}.experts.{x}.w1.weight", (i, w)),
+                        ParamSpec(f"{self.name}.experts.{x}.w2.weight", (w, i))]
+            return out
+
+        def load(self, tensors, runtime):
+            self.router = tensors[f"{self.name}.router.weight"].float()
+            self.w1 = torch.stack([tensors[f"{self.name}.experts.{x}.w1.weight"] for x in range(self.spec.experts)]).float()
+            self.w2 = torch.stack([tensors[f"{self.name}.experts.{x}.w2.weight"] for x in range(self.spec.experts)]).float()
+
+        def forward(self, ctx, x):
+            xf = x.float()
+            probs = torch.softmax(xf @ self.router.t(), dim=-1)  # router logits in float32
+            weight, expert = probs.max(dim=-1)
+            out = torch.zeros_like(xf)
+            for e in range(self.spec.experts):
+                rows = (expert == e).nonzero().flatten()
+                if rows.numel():
+                    h = torch.relu(xf[rows] @ self.w1[e].t())
+                    out[rows] = (h @ self.w2[e].t()) * weight[rows, None]
+            return out.to(x.dtype)
+
+    register_ffn("toy_top1", Top1Experts)
+
+
+def test_toy_routed_feed_forward_in_one_layer_of_two():
+    """One layer keeps the dense feed-forward, the other routes each token to one of
+    three experts: layers of one model choose their parts independently."""
+    define_toy_routed_ffn()
+    base = small_spec()
+    routed = replace(base.blocks[0], ffn=Top1Spec(experts=3, inner=40), ffn_name="moe")
+    spec = replace(base, blocks=(routed, base.blocks[1]))
+    w = cpu_weights(spec, seed=6)
+    assert "model.layers.0.moe.experts.2.w2.weight" in w and "model.layers.0.mlp.gate_proj.weight" not in w
+    runner, model, cache = make_runner(spec, w)
+
+    def want_for(ids):
+        cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
+        wd = {k: v.double() for k, v in w.items()}
+        n = len(ids)
+        cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+        x = wd["model.embed_tokens.weight"][torch.tensor(ids)]
+        p = "model.layers.0"
+        x = x + plain.attention_block(cfg, wd, f"{p}.self_attn", plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5), cos, sin, None)
+        h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
+        probs = torch.softmax(h @ wd[f"{p}.moe.router.weight"].t(), dim=-1)
+        ys = []
+        for t in range(n):
+            e = int(probs[t].argmax())
+            inner = torch.relu(wd[f"{p}.moe.experts.{e}.w1.weight"] @ h[t])
+            ys.append(probs[t, e] * (wd[f"{p}.moe.experts.{e}.w2.weight"] @ inner))
+        x = x + torch.stack(ys)
+        x = plain.decoder_layer(cfg, wd, 1, x, cos, sin)
+        return plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+    ids = torch.randint(0, 97, (23,), generator=torch.Generator().manual_seed(8)).tolist()
+    want = want_for(ids)
+    assert plain.rel_err(step_whole(runner, cache, ids), want) <= 1e-5
+    assert plain.rel_err(step_whole(runner, cache, ids, [5, 1, 1, 2, 14]), want) <= 1e-5
+
+
+# --------------------------------------------------- another position encoding
+
+
+@dataclass(frozen=True)
+class PairRotarySpec:
+    """Rotation of neighbouring pairs (2i, 2i + 1) by the angle pos * theta^(-2i/d)."""
+
+    kind: ClassVar[str] = "toy_pair_rotary"
+    theta: float
+
+
+def define_toy_position():
+    from shrike_amd.parts import PositionEncoding, register_position
+
+    class PairRotary(PositionEncoding):
+        def load(self, tensors, runtime):
+            self.device = runtime.device
+
+        def apply(self, ctx, qkv, heads, kv_heads, head_dim):
+            n = qkv.shape[0]
+            inv = 1.0 / (self.spec.theta ** (torch.arange(0, head_dim, 2, device=self.device).float() / head_dim))
+            angle = ctx.positions[:n].float()[:, None] * inv[None, :]
+            cos, sin = angle.cos()[:, None, :], angle.sin()[:, None, :]
+            qk = qkv[:, : (heads + kv_heads) * head_dim].view(n, heads + kv_heads, head_dim // 2, 2).float()
+            a, b = qk[..., 0], qk[..., 1]
+            rotated = torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1)
+            qkv[:, : (heads + kv_heads) * head_dim] = rotated.view(n, -1).to(qkv.dtype)
+
+    register_position("toy_pair_rotary", PairRotary)
+
+
+def test_toy_position_encoding_through_the_unfused_path():
+    """A position encoding without a fused kernel encodes q and k in place before
+    the keys go into the cache; decoding one by one gives what the whole prompt gives."""
+    define_toy_position()
+    base = small_spec()
+    blocks = tuple(replace(b, mixer=replace(b.mixer, position=PairRotarySpec(theta=500.0))) for b in base.blocks)
+    spec = replace(base, blocks=blocks)
+    w = cpu_weights(spec, seed=7)
+    runner, model, cache = make_runner(spec, w)
+
+    def pair_rope(x, positions):
+        d = x.shape[-1]
+        inv = 1.0 / (500.0 ** (torch.arange(0, d, 2).double() / d))
+        ang = positions.double()[:, None] * inv[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        a, b = x[..., 0::2], x[..., 1::2]
+        return torch.stack([a * cos - b * sin, b * cos + a * sin], dim=-1).flatten(-2)
+
+    def want_for(ids):
+        wd = {k: v.double() for k, v in w.items()}
+        n = len(ids)
+        pos = torch.arange(n)
+        x = wd["model.embed_tokens.weight"][torch.tensor(ids)]
+        for i in range(2):
+            p = f"model.layers.{i}"
+            h = plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5)
+            q = plain.linear(h, wd[f"{p}.self_attn.q_proj.weight"], wd[f"{p}.self_attn.q_proj.bias"]).view(n, 4, 16)
+            k = plain.linear(h, wd[f"{p}.self_attn.k_proj.weight"], wd[f"{p}.self_attn.k_proj.bias"]).view(n, 2, 16)
+            v = plain.linear(h, wd[f"{p}.self_attn.v_proj.weight"], wd[f"{p}.self_attn.v_proj.bias"]).view(n, 2, 16)
+            att = plain.causal_attention(pair_rope(q, pos), pair_rope(k, pos), v)
+            x = x + plain.linear(att.reshape(n, -1), wd[f"{p}.self_attn.o_proj.weight"])
+            h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
+            x = x + plain.swiglu(h, wd[f"{p}.mlp.gate_proj.weight"], wd[f"{p}.mlp.up_proj.weight"], wd[f"{p}.mlp.down_proj.weight"])
+        return plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+    ids = torch.randint(0, 97, (21,), generator=torch.Generator().manual_seed(9)).tolist()
+    want = want_for(ids)
+    assert plain.rel_err(step_whole(runner, cache, ids), want) <= 1e-5
+    assert plain.rel_err(step_whole(runner, cache, ids, [9] + [1] * 12), want) <= 1e-5
