@@ -426,6 +426,9 @@ __global__ void __launch_bounds__(WAVES* kWave)
 // the loads of the next two stages are in flight (in registers) while a stage is
 // multiplied.
 
+constexpr int kDies = 8;        // accelerator dies (XCDs), each with an L2 of its own
+constexpr int kDieUnits = 32;  // compute units per die
+
 // GM x GN wavefronts per workgroup, each with WM x WN MFMA tiles (16 x 16): the
 // workgroup covers 16*GM*WM weight rows x 16*GN*WN tokens.  KS: MFMA steps (32 of
 // k) per stage.  The stages live in dynamic LDS, [buffer][fragment][lane].
@@ -435,7 +438,7 @@ __global__ void __launch_bounds__(GM* GN* kWave)
     gemm_big_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                     const uint4* __restrict__ wt, int ktiles, int m,
                     const float* __restrict__ bias, void* __restrict__ out, int ldo, int out_f32,
-                    int accumulate, int vec, int ksplit) {
+                    int accumulate, int vec, int ksplit, int tiles_x, int tiles_y, int by_die) {
   constexpr int kWaves = GM * GN;
   constexpr int kWFrags = GM * WM * KS, kAFrags = GN * WN * KS;  // fragments per stage
   constexpr int kFrags = kWFrags + kAFrags;
@@ -443,15 +446,32 @@ __global__ void __launch_bounds__(GM* GN* kWave)
   auto stage = [&](int buf, int frag) -> uint4* { return stage_mem + (buf * kFrags + frag) * kWave; };
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wm = wave / GN, wn = wave % GN;  // place of the wavefront in the workgroup's tile
-  const int mb0 = blockIdx.x * (GM * WM);  // first block of 16 weight rows
-  const int tok0 = blockIdx.y * (16 * GN * WN);
+  // Which tile: workgroups are handed to the chip's eight dies (each with its own
+  // L2) in turn, workgroup p to die p % 8.  The tiles are therefore dealt out in
+  // blocks of 32 (up to 8 token tiles of 32 / that many weight tiles) and block B goes to
+  // die B % 8, whose 32 compute units then work on tiles that share their
+  // operands: the die's L2 serves most of their loads.
+  // With too few tiles for that (by_die == 0) they are taken in plain order.
+  int tile_x = blockIdx.x % tiles_x, tile_y = blockIdx.x / tiles_x;
+  if (by_die) {
+    const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
+    const int block_y = tiles_y < 8 ? tiles_y : 8, block_x = kDieUnits / block_y;
+    const int blocks_x = (tiles_x + block_x - 1) / block_x;
+    const int block = (turn / kDieUnits) * kDies + die, within = turn % kDieUnits;
+    tile_x = (block % blocks_x) * block_x + within / block_y;
+    tile_y = (block / blocks_x) * block_y + within % block_y;
+    if (within >= block_x * block_y) return;
+  }
+  if (tile_x >= tiles_x || tile_y >= tiles_y) return;
+  const int mb0 = tile_x * (GM * WM);  // first block of 16 weight rows
+  const int tok0 = tile_y * (16 * GN * WN);
   // blocks of 16 weight rows; a gated weight has two per 16 output rows
   const int mblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
-  // blockIdx.z: which share of the k stages (ksplit workgroups per tile leave float32
+  // blockIdx.y: which share of the k stages (ksplit workgroups per tile leave float32
   // partial sums [ksplit][n][m] that the reading kernel adds up)
   const int all_stages = (ktiles + KS - 1) / KS;
   const int per_split = (all_stages + ksplit - 1) / ksplit;
-  const int st_first = blockIdx.z * per_split;
+  const int st_first = blockIdx.y * per_split;
   const int nstages = st_first + per_split < all_stages ? st_first + per_split : all_stages;
 
   f32x4 acc[WM][WN];
@@ -615,7 +635,7 @@ __global__ void __launch_bounds__(GM* GN* kWave)
         v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r] : acc[i][jn][r];
         if (bias && row0 + r < m) v[r] += bias[row0 + r];
       }
-      const size_t idx = (static_cast<size_t>(blockIdx.z) * n + token) * ldo + row0;
+      const size_t idx = (static_cast<size_t>(blockIdx.y) * n + token) * ldo + row0;
       if (out_f32) {
         float* o = static_cast<float*>(out) + idx;
 #pragma unroll
@@ -701,21 +721,30 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
                        int m, const float* bias, void* out, int ldo, int of, int accumulate, int vec,
                        int gated, int wblocks, int ksplit) {
   constexpr int lds = 2 * (GM * WM + GN * WN) * KS * kWave * 16;
-  dim3 grid((wblocks + GM * WM - 1) / (GM * WM), (n + 16 * GN * WN - 1) / (16 * GN * WN), ksplit);
+  const int tiles_x = (wblocks + GM * WM - 1) / (GM * WM), tiles_y = (n + 16 * GN * WN - 1) / (16 * GN * WN);
+  // one-dimensional, in whole rounds of the eight dies' blocks of 32 tiles (see the kernel)
+  const int block_y = tiles_y < 8 ? tiles_y : 8, block_x = kDieUnits / block_y;
+  const long long blocks = static_cast<long long>((tiles_x + block_x - 1) / block_x) *
+                           ((tiles_y + block_y - 1) / block_y);
+  // worth it from four rounds of workgroups on: below that, whole dies would stay idle
+  const int by_die = static_cast<long long>(tiles_x) * tiles_y >= 4 * kDies * kDieUnits;
+  dim3 grid(by_die ? static_cast<unsigned>((blocks + kDies - 1) / kDies * kDies * kDieUnits)
+                   : static_cast<unsigned>(tiles_x * tiles_y),
+            ksplit);
   if (gated) {
     auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, true>;
     if (lds > 65536)
       hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate,
-                                              vec, ksplit);
+                                              vec, ksplit, tiles_x, tiles_y, by_die);
   } else {
     auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, false>;
     if (lds > 65536)
       hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                           hipFuncAttributeMaxDynamicSharedMemorySize, lds);
     kernel<<<grid, GM * GN * kWave, lds, s>>>(ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate,
-                                              vec, ksplit);
+                                              vec, ksplit, tiles_x, tiles_y, by_die);
   }
 }
 
