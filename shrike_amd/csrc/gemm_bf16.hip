@@ -795,15 +795,24 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   if (n > 64) {
     SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
     const int wblocks = (gated ? 2 : 1) * mb;  // blocks of 16 weight rows
-    // Tile of the workgroup: the largest of 256 x 256, 256 x 128 and 128 x 128
-    // (weight rows x tokens) that still gives every compute unit a workgroup.
-    auto tiles = [&](int rows, int tokens) {
-      return static_cast<long long>((wblocks * 16 + rows - 1) / rows) * ((n + tokens - 1) / tokens);
+    // Tile of the workgroup: 256 x 256, 256 x 128 or 128 x 128 (weight rows x
+    // tokens), whichever finishes first by this estimate: rounds of workgroups
+    // over the chip (256 compute units; two of the smallest tile fit on one) times
+    // the tile's work over the rate a workgroup of that shape was measured at.
+    auto rounds = [&](int rows, int tokens, int slots) {
+      const long long tiles =
+          static_cast<long long>((wblocks * 16 + rows - 1) / rows) * ((n + tokens - 1) / tokens);
+      return static_cast<double>((tiles + slots - 1) / slots);
     };
-    if (ksplit == 1 && tiles(256, 256) >= 256)
+    const double cost_a = rounds(256, 256, 256) * (256.0 * 256.0) / 4.2;
+    const double cost_b = rounds(256, 128, 256) * (256.0 * 128.0) / 3.4;
+    // the smallest tile runs faster while it has its compute unit to itself
+    const bool c_alone = rounds(128, 128, 256) <= 1.0;
+    const double cost_c = rounds(128, 128, 512) * (128.0 * 128.0) / (c_alone ? 2.6 : 1.5);
+    if (ksplit == 1 && cost_a <= cost_b && cost_a <= cost_c)
       launch_big<4, 2, 4, 8, 1>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
-    else if (ksplit == 1 && tiles(256, 128) >= 200)
+    else if (ksplit == 1 && cost_b <= cost_c)
       launch_big<4, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
     else
