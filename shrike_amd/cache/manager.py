@@ -3,8 +3,8 @@ one pool per group of layers with the same need, and slots for per-request
 state of fixed size.
 
 Layers whose mixers ask for the same PagedKVSpec form a group; a group has its
-own pool of pages, its own device tensors (keys
-``[layers, pages, kv_heads, page_size, head_dim]``; values transposed,
+own pool of pages, its own device tensors (keys in slabs of 32 elements,
+``[layers, pages, kv_heads, head_dim / 32, page_size, 32]``; values transposed,
 ``[layers, pages, kv_heads, head_dim, page_size]``, so that the keys of a page
 are contiguous for every element) and, per request, its own block table.  A
 group with a window gives pages back as soon as no later query
@@ -126,8 +126,11 @@ class CacheManager:
             s = g.spec
             # one page more than the pool hands out: page `num_pages` is where the
             # padding rows of a fixed-size (graph) batch put their keys and values
+            # keys of a page and head in slabs of 32 elements (whole rows where the head
+            # size is no multiple of 32): what the attention kernels' operand loads want
+            slab = 32 if s.head_dim % 32 == 0 else s.head_dim
             g.k_tensor = torch.zeros(
-                len(g.layers), self.num_pages + 1, s.num_kv_heads, self.page_size, s.head_dim,
+                len(g.layers), self.num_pages + 1, s.num_kv_heads, s.head_dim // slab, self.page_size, slab,
                 dtype=dtype, device=device,
             )
             g.v_tensor = torch.zeros(

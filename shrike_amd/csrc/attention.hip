@@ -54,9 +54,15 @@ __global__ void __launch_bounds__(kAttnThreads)
       const int page = table[j / page_size];
       if (page >= 0 && page < num_pages) {
         row = (page * kv_heads + kvh) * page_size + j % page_size;
-        const T* kr = k_pool + static_cast<size_t>(row) * head_dim;
+        // keys are stored in slabs: [head_dim / slab][page_size][slab] per page and head
+        const int slab = key_slab(head_dim);
+        const T* kr = k_pool + static_cast<size_t>(page * kv_heads + kvh) * page_size * head_dim +
+                      static_cast<size_t>(j % page_size) * slab;
         float dot = 0.f;
-        for (int e = 0; e < head_dim; ++e) dot = fmaf(qs[e], to_float(kr[e]), dot);
+        for (int e0 = 0; e0 < head_dim; e0 += slab) {
+          for (int e = 0; e < slab; ++e) dot = fmaf(qs[e0 + e], to_float(kr[e]), dot);
+          kr += static_cast<size_t>(page_size) * slab;
+        }
         s = dot * scale;
       }
     }

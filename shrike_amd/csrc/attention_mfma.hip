@@ -6,7 +6,8 @@
 // (padded to 16).  The wavefront walks its key range in chunks of 32 keys:
 //
 //   S = Q K^T      two 16x16 tiles, v_mfma_f32_16x16x32_bf16 over head_dim;
-//                  K rows are read straight from the page ([slot][head_dim])
+//                  K rows are read straight from the page (slabs of 32 elements:
+//                  [head_dim / 32][slot][32], 64 bytes per key and slab)
 //   softmax        running maximum and sum per row in float32, exp in float32
 //   O += P V       P goes through LDS into operand layout; V is stored
 //                  transposed in the cache ([head_dim][slot]), so 8 keys of one
@@ -79,7 +80,7 @@ __device__ __forceinline__ int page_at(const PageWindow& w, int entry) {
 
 struct TileArgs {
   const int32_t* table;  // block table of the sequence
-  const bf16* k_pool;    // [pages][kv_heads][page_size][D]
+  const bf16* k_pool;    // [pages][kv_heads][D / 32][page_size][32]
   const bf16* v_pool;    // [pages][kv_heads][D][page_size]
   int page_size;
   int kv_heads;
@@ -113,12 +114,12 @@ __device__ __forceinline__ void load_chunk(Chunk<D>& c, const TileArgs& ta, cons
     if (live) {
       const int page = kpage;
       krow = ta.k_pool + (static_cast<size_t>(page) * ta.kv_heads + ta.kvh) * head_elems +
-             static_cast<size_t>(key0 % ps + j) * D + kg * 8;
+             static_cast<size_t>(key0 % ps + j) * 32 + kg * 8;  // slab ds follows at ds * ps * 32
     }
 #pragma unroll
     for (int ds = 0; ds < D / 32; ++ds) {
       c.k[tt][ds].u = make_uint4(0, 0, 0, 0);
-      if (live) c.k[tt][ds].u = *reinterpret_cast<const uint4*>(krow + ds * 32);
+      if (live) c.k[tt][ds].u = *reinterpret_cast<const uint4*>(krow + static_cast<size_t>(ds) * ps * 32);
     }
   }
   // this lane supplies keys kb + 8*kg .. +8 of element db*16 + j
@@ -355,7 +356,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
     const bool k_second = j >= 8;
     int k_lane[2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) k_lane[t] = (8 * ((j / 4) % 2) + 4 * t + j % 4) * D + g * 8;
+    for (int t = 0; t < 2; ++t) k_lane[t] = (8 * ((j / 4) % 2) + 4 * t + j % 4) * 32 + g * 8;
     const bool v_second = g >= 2;
     const int v_lane = j * page_size + 8 * (g % 2);
     const size_t head_elems = static_cast<size_t>(page_size) * D;  // one kv head of one page
@@ -371,13 +372,15 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
       const size_t head_a = (static_cast<size_t>(page_a) * kv_heads + kvh) * head_elems;
       const size_t head_c = (static_cast<size_t>(page_c) * kv_heads + kvh) * head_elems;
       const int slot_a = pd.mod(kb), slot_c = pd.mod(kb + 16);
-      const bf16* krow = k_pool + (k_second ? head_c + static_cast<size_t>(slot_c) * D
-                                            : head_a + static_cast<size_t>(slot_a) * D);
+      // keys lie in slabs of 32 elements, [D / 32][page_size][32]
+      const bf16* krow = k_pool + (k_second ? head_c + static_cast<size_t>(slot_c) * 32
+                                            : head_a + static_cast<size_t>(slot_a) * 32);
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int ds = 0; ds < D / 32; ++ds)
-          c.k[t][ds].u = *reinterpret_cast<const uint4*>(krow + k_lane[t] + ds * 32);
+          c.k[t][ds].u = *reinterpret_cast<const uint4*>(krow + k_lane[t] +
+                                                         static_cast<size_t>(ds) * page_size * 32);
       const bf16* vcol = v_pool + (v_second ? head_c + slot_c : head_a + slot_a) + v_lane;
 #pragma unroll
       for (int db = 0; db < D / 16; ++db)
@@ -766,7 +769,7 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
     is_k[i] = f < kKFrags;
     if (is_k[i]) {
       const int t = f / (D / 32), ds = f % (D / 32);
-      lane_off[i] = (8 * ((j / 4) % 2) + 4 * t + j % 4) * D + ds * 32 + g * 8;
+      lane_off[i] = (8 * ((j / 4) % 2) + 4 * t + j % 4) * 32 + ds * page_size * 32 + g * 8;
     } else {
       const int db = f - kKFrags;
       lane_off[i] = (db * 16 + j) * page_size + 8 * (g % 2);
@@ -782,8 +785,8 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
     const size_t head_a = (static_cast<size_t>(page_a) * kv_heads + kvh) * head_elems;
     const size_t head_c = (static_cast<size_t>(page_c) * kv_heads + kvh) * head_elems;
     const int slot_a = pd.mod(kb), slot_c = pd.mod(kb + 16);
-    const bf16* krow = k_pool + (second_k ? head_c + static_cast<size_t>(slot_c) * D
-                                          : head_a + static_cast<size_t>(slot_a) * D);
+    const bf16* krow = k_pool + (second_k ? head_c + static_cast<size_t>(slot_c) * 32
+                                          : head_a + static_cast<size_t>(slot_a) * 32);
     const bf16* vcol = v_pool + (second_v ? head_c + slot_c : head_a + slot_a);
 #pragma unroll
     for (int i = 0; i < kPer; ++i)

@@ -76,6 +76,21 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return total;
 }
 
+// ------------------------------------------------------- layout of cached keys
+// The keys of one key/value head in one page are stored in slabs of 32
+// elements, [head_dim / 32][page_size][32] (the whole row as one slab where
+// head_dim is no multiple of 32): the 16 bytes a lane of an MFMA operand needs
+// from each of four consecutive keys then lie side by side, 64 bytes per key,
+// and a wavefront's operand load touches whole cache lines.  Values are stored
+// transposed, [head_dim][page_size].
+__host__ __device__ inline int key_slab(int head_dim) { return head_dim % 32 == 0 ? 32 : head_dim; }
+
+// Offset of element d of the key in `slot`, in elements from the start of its page's head.
+__host__ __device__ inline size_t key_offset(int slot, int d, int page_size, int head_dim) {
+  const int slab = key_slab(head_dim);
+  return (static_cast<size_t>(d / slab) * page_size + slot) * slab + d % slab;
+}
+
 // ---------------------------------------------------------------- host side
 
 enum DType : int { kF32 = 0, kBF16 = 1 };

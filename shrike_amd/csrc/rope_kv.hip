@@ -93,7 +93,7 @@ __global__ void __launch_bounds__(kRopeThreads)
     if (page < 0 || page >= num_pages) page = -1;
   }
   const int slot = pos % page_size;
-  // keys [page][kv head][slot][head_dim]; values transposed [page][kv head][head_dim][slot]
+  // keys [page][kv head] in slabs (key_offset); values transposed [page][kv head][head_dim][slot]
   const size_t page_base = static_cast<size_t>(page < 0 ? 0 : page) * kv_heads * page_size * head_dim;
 
   for (int f = threadIdx.x; f < half; f += kRopeThreads) {
@@ -117,16 +117,16 @@ __global__ void __launch_bounds__(kRopeThreads)
       row[col] = from_float<T>(o1);
       row[col + half] = from_float<T>(o2);
     } else if (page >= 0) {
-      T* dst = k_pool + page_base + (static_cast<size_t>(h - heads) * page_size + slot) * head_dim;
-      dst[i] = from_float<T>(o1);
-      dst[i + half] = from_float<T>(o2);
+      T* dst = k_pool + page_base + static_cast<size_t>(h - heads) * page_size * head_dim;
+      dst[key_offset(slot, i, page_size, head_dim)] = from_float<T>(o1);
+      dst[key_offset(slot, i + half, page_size, head_dim)] = from_float<T>(o2);
     }
   } else if (role == kTailItem) {
     if (h < heads) {
       row[col] = from_float<T>(x1);
     } else if (page >= 0) {
-      k_pool[page_base + (static_cast<size_t>(h - heads) * page_size + slot) * head_dim + i] =
-          from_float<T>(x1);
+      k_pool[page_base + static_cast<size_t>(h - heads) * page_size * head_dim +
+             key_offset(slot, i, page_size, head_dim)] = from_float<T>(x1);
     }
   } else if (role == kValueItem) {
     if (page >= 0) v_pool[page_base + static_cast<size_t>(i) * page_size + slot] = from_float<T>(x1);

@@ -196,12 +196,23 @@ def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, g
     )
 
 
+def key_slab(head_dim: int) -> int:
+    """Elements per slab of the cached keys: 32, or the whole row where head_dim
+    is no multiple of 32 (csrc/common.h: key_slab)."""
+    return 32 if head_dim % 32 == 0 else head_dim
+
+
+def key_pool_shape(pages: int, kv_heads: int, page_size: int, head_dim: int) -> tuple:
+    """Keys of a page and head lie in slabs: [pages, kv_heads, head_dim / slab, page_size, slab]."""
+    slab = key_slab(head_dim)
+    return (pages, kv_heads, head_dim // slab, page_size, slab)
+
+
 def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size) -> None:
-    """Keys [pages, kv_heads, page_size, head_dim]; values transposed
-    [pages, kv_heads, head_dim, page_size]."""
+    """Keys in slabs (key_pool_shape); values transposed [pages, kv_heads, head_dim, page_size]."""
     pages = k_pool.shape[0]
-    if tuple(k_pool.shape) != (pages, kv_heads, page_size, head_dim):
-        raise KernelError(f"{who}: key pool must be [pages, {kv_heads}, {page_size}, {head_dim}], "
+    if tuple(k_pool.shape) != key_pool_shape(pages, kv_heads, page_size, head_dim):
+        raise KernelError(f"{who}: key pool must be {list(key_pool_shape('pages', kv_heads, page_size, head_dim))}, "
                           f"got {tuple(k_pool.shape)}")
     if tuple(v_pool.shape) != (pages, kv_heads, head_dim, page_size):
         raise KernelError(f"{who}: value pool must be [pages, {kv_heads}, {head_dim}, {page_size}], "

@@ -135,7 +135,8 @@ def paged_setup(seq_lens, page_size, num_pages, kv_heads, head_dim, dtype, seed=
     for n in seq_lens:
         need = -(-n // page_size)
         tables.append([perm.pop() for _ in range(need)] + [0] * (width - need))
-    k_pool = torch.full((num_pages, kv_heads, page_size, head_dim), float("nan"), dtype=dtype, device="cuda")
+    slab = 32 if head_dim % 32 == 0 else head_dim
+    k_pool = torch.full((num_pages, kv_heads, head_dim // slab, page_size, slab), float("nan"), dtype=dtype, device="cuda")
     v_pool = torch.full((num_pages, kv_heads, head_dim, page_size), float("nan"), dtype=dtype, device="cuda")
     return torch.tensor(tables, dtype=torch.int32, device="cuda"), k_pool, v_pool
 
@@ -164,12 +165,21 @@ def test_rope_kv_store(ops, dtype, heads, kv_heads, head_dim, page_size, theta):
     for t in range(n):
         s, p = int(token_seq[t]), int(positions[t])
         page = int(tables[s, p // page_size])
-        close(k_pool[page, :, p % page_size], plain.apply_rope(k[t : t + 1], cos[t : t + 1], sin[t : t + 1])[0], dtype)
+        close(get_key(k_pool, page, p % page_size), plain.apply_rope(k[t : t + 1], cos[t : t + 1], sin[t : t + 1])[0], dtype)
         assert torch.equal(v_pool[page, :, :, p % page_size].cpu().double(), v[t])
     # nothing else was written: every other slot is still NaN
     written = sum(seq_lens) * kv_heads * head_dim
     assert int((~torch.isnan(k_pool.float())).sum()) == written
     assert int((~torch.isnan(v_pool.float())).sum()) == written
+
+
+def put_key(k_pool, page, slot, k):
+    """k [kv_heads, head_dim] into the slabs of a page: [kv_heads, head_dim / slab, page_size, slab]."""
+    k_pool[page, :, :, slot, :] = k.to(k_pool.device).view(k_pool.shape[1], k_pool.shape[2], k_pool.shape[4])
+
+
+def get_key(k_pool, page, slot):
+    return k_pool[page, :, :, slot, :].reshape(k_pool.shape[1], -1)
 
 
 def reference_attention(q, k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale):
@@ -180,7 +190,8 @@ def reference_attention(q, k_pool, v_pool, tables, seq_lens, starts, page_size, 
     for s, (start, n_new) in enumerate(zip(starts, seq_lens)):
         ctx = start + n_new
         pages = tables[s, : -(-ctx // page_size)].long().cpu()
-        k = k_pool.cpu().double()[pages].permute(0, 2, 1, 3).reshape(-1, k_pool.shape[1], k_pool.shape[3])[:ctx]
+        # [pages, kv_heads, slabs, page_size, slab] -> [keys, kv_heads, head_dim]
+        k = k_pool.cpu().double()[pages].permute(0, 3, 1, 2, 4).reshape(-1, k_pool.shape[1], k_pool.shape[2] * k_pool.shape[4])[:ctx]
         v = v_pool.cpu().double()[pages].permute(0, 3, 1, 2).reshape(-1, v_pool.shape[1], v_pool.shape[2])[:ctx]
         k, v = torch.nan_to_num(k), torch.nan_to_num(v)  # slots outside the window may be poisoned
         full_q = torch.zeros(ctx, heads, q.shape[2], dtype=torch.float64)
@@ -209,7 +220,7 @@ def test_attention_mixed_batch(ops, dtype, heads, kv_heads, head_dim, page_size,
     for s, c in enumerate(ctx):  # fill each sequence's slots; everything else stays NaN
         for p in range(c):
             page = int(tables[s, p // page_size])
-            k_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
+            put_key(k_pool, page, p % page_size, torch.randn(kv_heads, head_dim).to(dtype))
             v_pool[page, :, :, p % page_size] = torch.randn(kv_heads, head_dim).to(dtype)
     n = sum(seq_lens)
     q = torch.randn(n, heads, head_dim).to(dtype)
@@ -236,7 +247,7 @@ def test_attention_finds_one_far_key_among_hundreds(ops, dtype):
     k[far] = q[0, ::2] * 4.0  # heads 0 and 2 are the first of each group
     for p in range(ctx):
         page = int(tables[0, p // page_size])
-        k_pool[page, :, p % page_size] = k[p].to(dtype)
+        put_key(k_pool, page, p % page_size, k[p].to(dtype))
         v_pool[page, :, :, p % page_size] = v[p].to(dtype)
     out = torch.empty(1, heads * head_dim, device="cuda", dtype=dtype)
     ops.attention(dev(q, dtype).view(1, -1), out, heads, kv_heads, head_dim, torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"),
@@ -261,7 +272,7 @@ def test_attention_window_edge(ops, dtype):
     k[edge + 1] = q[0] * 0.5
     for p in range(ctx):
         page = int(tables[0, p // page_size])
-        k_pool[page, :, p % page_size] = k[p].to(dtype)
+        put_key(k_pool, page, p % page_size, k[p].to(dtype))
         v_pool[page, :, :, p % page_size] = v[p].to(dtype)
     args = (heads, kv_heads, head_dim, torch.tensor([ctx - 1], dtype=torch.int32, device="cuda"),
             torch.zeros(1, dtype=torch.int32, device="cuda"), tables, k_pool, v_pool, page_size)
@@ -280,7 +291,7 @@ def test_attention_refuses_head_sizes_it_cannot_do(ops):
 
     with pytest.raises(KernelError, match="head_dim"):
         z = torch.zeros(1, 272, device="cuda")
-        k_pool = torch.zeros(2, 1, 4, 272, device="cuda")
+        k_pool = torch.zeros(2, 1, 1, 4, 272, device="cuda")
         v_pool = torch.zeros(2, 1, 272, 4, device="cuda")
         i = torch.zeros(1, dtype=torch.int32, device="cuda")
         ops.attention(z, torch.empty_like(z), 1, 1, 272, i, i, i.view(1, 1), k_pool, v_pool, 4, None, 1.0)
@@ -417,11 +428,11 @@ def test_gemm_tiled_weight_rows_do_not_depend_on_the_rest_of_the_batch(ops):
 
 
 def fill_pools(tables, k_pool, v_pool, ctx, page_size):
-    kv_heads, head_dim = k_pool.shape[1], k_pool.shape[3]
+    kv_heads, head_dim = v_pool.shape[1], v_pool.shape[2]
     for s, c in enumerate(ctx):
         for p in range(c):
             page = int(tables[s, p // page_size])
-            k_pool[page, :, p % page_size] = torch.randn(kv_heads, head_dim).to(k_pool.dtype)
+            put_key(k_pool, page, p % page_size, torch.randn(kv_heads, head_dim).to(k_pool.dtype))
             v_pool[page, :, :, p % page_size] = torch.randn(kv_heads, head_dim).to(v_pool.dtype)
 
 
@@ -500,7 +511,7 @@ def test_attention_mfma_finds_one_far_key_among_thousands(ops):
     k[far, 0] = q[0, 3] * 2.0  # head 3 of group 0
     for p in range(ctx):
         page = int(tables[0, p // page_size])
-        k_pool[page, :, p % page_size] = k[p].to(dtype)
+        put_key(k_pool, page, p % page_size, k[p].to(dtype))
         v_pool[page, :, :, p % page_size] = v[p].to(dtype)
     out = torch.empty(1, heads * head_dim, device="cuda", dtype=dtype)
     partial = torch.empty(heads * 16 * (head_dim + 2), device="cuda")
@@ -586,7 +597,7 @@ def test_rope_kv_store_adds_up_a_split_product(ops):
     for t in range(n):
         p = int(positions[t])
         page = int(tables[t, p // page_size])
-        close(k_pool[page, :, p % page_size], k[t], dtype)
+        close(get_key(k_pool, page, p % page_size), k[t], dtype)
         close(v_pool[page, :, :, p % page_size], v[t], dtype)
 
 
