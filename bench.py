@@ -1,6 +1,6 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b]
 
 The model has the layer sizes of the Qwen2.5-7B shape (28 layers, hidden 3584,
 28 query heads over 4 key/value heads of 128, intermediate 18944, vocabulary
@@ -43,6 +43,14 @@ SHAPE_7B = {
     "max_position_embeddings": 32768,
     "eos_token_id": 151645,
     "torch_dtype": "bfloat16",
+}
+# the other shapes of the Qwen2.5 family that the engine is sized for: what differs from 7B
+SHAPES = {
+    "7b": {},
+    "14b": {"hidden_size": 5120, "intermediate_size": 13824, "num_hidden_layers": 48,
+            "num_attention_heads": 40, "num_key_value_heads": 8, "rms_norm_eps": 1e-5},
+    "32b": {"hidden_size": 5120, "intermediate_size": 27648, "num_hidden_layers": 64,
+            "num_attention_heads": 40, "num_key_value_heads": 8, "rms_norm_eps": 1e-5},
 }
 PROMPT_LEN = 2048
 CONTEXT_END = 4096
@@ -162,6 +170,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=SHAPE_7B["num_hidden_layers"],
                     help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b",
+                    help="layer sizes: Qwen2.5-7B (the default and the reported figure), 14B or 32B")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -180,7 +190,10 @@ def main() -> int:
     import shrike_amd.models  # noqa: F401
     from shrike_amd.models.qwen2 import Qwen2Config, build_spec
 
-    raw = dict(SHAPE_7B, num_hidden_layers=args.layers)
+    raw = dict(SHAPE_7B, **SHAPES[args.shape])
+    layers_of_config = raw["num_hidden_layers"]
+    if args.layers != SHAPE_7B["num_hidden_layers"] or args.shape == "7b":
+        raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
@@ -197,7 +210,7 @@ def main() -> int:
 
     main_run = results[args.batch]
     line = {
-        "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-7B shape, 2048-token prompts, "
+        "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-{args.shape.upper()} shape, 2048-token prompts, "
                   "decode to 4096)",
         "value": round(main_run["tok_s"], 1),
         "unit": "tok/s",
@@ -211,9 +224,9 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic: random weights N(0, 0.02), prompt ids uniform in [0, vocab)",
         "config": {
-            "model": "Qwen2.5-7B shape (Qwen2ForCausalLM)",
+            "model": f"Qwen2.5-{args.shape.upper()} shape (Qwen2ForCausalLM)",
             "layers": cfg.num_hidden_layers,
-            "layers_of_config": SHAPE_7B["num_hidden_layers"],
+            "layers_of_config": layers_of_config,
             "hidden": cfg.hidden_size,
             "heads": cfg.num_attention_heads,
             "kv_heads": cfg.num_key_value_heads,
