@@ -272,3 +272,47 @@ def test_graph_replays_equal_eager_steps(dtype, model_root):
     assert len(eager) == len(graphed)
     for a, b in zip(eager, graphed):
         assert torch.equal(a, b)
+
+
+def test_random_arrivals_under_page_pressure_with_shared_prefixes(model_root):
+    """Requests arrive while others run, share prefixes, differ in length and in
+    sampling, and the pool is small enough for preemptions: every greedy
+    request still produces what it produces alone in a roomy engine, and every
+    page and slot is back in the end."""
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+
+    model_dir = make_model_dir("B", model_root, mode="unit")
+    rng = random.Random(11)
+    stems = prompts_for("B", [24, 17], seed=12)
+    jobs = []
+    for i in range(14):
+        stem = stems[i % 2][: rng.choice([8, 16, 17, 24])] if i % 3 else []
+        tail = prompts_for("B", [rng.randint(1, 30)], seed=100 + i)[0]
+        greedy = i % 4 != 3
+        sp = SamplingParams(max_new_tokens=rng.randint(1, 25), ignore_eos=True,
+                            temperature=0.0 if greedy else 0.8, top_p=0.9, seed=i)
+        jobs.append((stem + tail, sp, greedy))
+
+    roomy = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=128,
+                      enable_prefix_caching=False)
+    want = [roomy.generate([p], sp)[0] for p, sp, _ in jobs]
+
+    tight = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=22,
+                      max_tokens_per_step=24, max_running=5)
+    got, ids, pending = {}, {}, list(range(len(jobs)))
+    while pending or tight.has_work:
+        for _ in range(rng.randint(0, 2)):  # zero to two arrivals before each step
+            if pending:
+                i = pending.pop(0)
+                ids[tight.add_request(jobs[i][0], jobs[i][1])] = i
+        for o in tight.step():
+            got.setdefault(ids[o.req_id], []).append(o.token_id)
+        tight.cache.check([r.cache for r in tight.scheduler.running if r.cache is not None])
+    assert tight.metrics()["preemptions"] > 0 and tight.metrics()["prefix_cache_hit_rate"] > 0
+    for i, (_, sp, greedy) in enumerate(jobs):
+        assert len(got[i]) == sp.max_new_tokens
+        if greedy:
+            assert got[i] == want[i], f"request {i}"
+    assert tight.cache.num_free == 22 and not tight.scheduler.running
+    tight.cache.check([])
