@@ -671,25 +671,26 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
 }
 
 // ------------------------------------------------- prefill, keys shared in LDS
-// A workgroup of 8 wavefronts serves every query head of one key/value head for
+// A workgroup of 16 wavefronts serves every query head of one key/value head for
 // a run of 16-query tiles of one sequence.  The chunk of 32 keys is fetched once
-// and staged in LDS in operand layout; a wavefront owns two "units" (query head,
-// query tile) and multiplies every fragment it reads from LDS with both.  The
-// softmax arithmetic, not the matrix unit, bounds a wavefront, and the workgroup
-// with the last queries sets the kernel's time, hence many wavefronts with
-// little each (four with four units measured 1.5 times slower).  Unit u < tiles *
-// group is tile u / group, head u % group of the key/value head.  The products
-// are formed transposed as in the decode kernel (S^T = K Q^T, O^T += V^T P^T):
-// a lane owns one query, and P needs no trip through LDS.
+// and staged in LDS in operand layout; a wavefront owns one "unit" (query head,
+// query tile) (the code allows several, which then share every fragment read
+// from LDS).  The softmax arithmetic, not the matrix unit, bounds a wavefront,
+// and the workgroup with the last queries sets the kernel's time, hence many
+// wavefronts with little each: for 2,048 queries of 28 heads over 4, sixteen
+// wavefronts with one unit take 96 us, eight with two 104 us, four with four 150
+// us.  Unit u < tiles * group is tile u / group, head u % group of the key/value
+// head.  The products are formed transposed as in the decode kernel (S^T = K Q^T,
+// O^T += V^T P^T): a lane owns one query, and P needs no trip through LDS.
 // grid (workgroup tiles, kv_heads); wg_seq / wg_q0 as tile_seq / tile_q0 above,
 // in steps of 16 * tiles queries.
 
-constexpr int kUnitsPerWave = 2;
-constexpr int kSharedWaves = 8;
+constexpr int kUnitsPerWave = 1;
+constexpr int kSharedWaves = 16;
 
 template <int D>
 __global__ void __launch_bounds__(kSharedWaves* kWave)
-    __attribute__((amdgpu_waves_per_eu(kUnitsPerWave <= 2 || kSharedWaves > 4 ? 2 : 1)))
+    __attribute__((amdgpu_waves_per_eu(kSharedWaves >= 16 ? 4 : 2)))
     attention_prefill_shared_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                                     int heads, int kv_heads, int tiles,
                                     const int32_t* __restrict__ cu_q,
@@ -755,7 +756,7 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
     for (int db = 0; db < D / 16; ++db) o[u][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- staging.  Wavefront w fetches fragments w, w + 4, ...  Fragment f < kKFrags
+  // ---- staging.  Wavefront w fetches fragments w, w + kSharedWaves, ...  Fragment f < kKFrags
   // is K tile f / (D/32), head_dim slice f % (D/32); row i of K tile t is key
   // 8*(i/4) + 4*t + i%4 of the chunk, so that lane (j, g) of a score tile ends up
   // with the eight keys 8*g .. 8*g + 7.  The others are V^T blocks of 16 elements.
