@@ -821,6 +821,22 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }
+  if (n > 32 && mb < 4096) {
+    // 33 to 64 tokens: the LDS-staged kernel with tiles of 256 weight rows x 64
+    // tokens beats the kernel below where it has at least half the chip's
+    // compute units to fill and a long walk along k for each workgroup (the
+    // 7B down and gate/up matrices at 64 tokens: 36 us against 46, 61 against 65)
+    const int wblocks = (gated ? 2 : 1) * mb;
+    const int workgroups = ((wblocks + 15) / 16) * ksplit;
+    const int stages = (kt / ksplit + 1) / 2;
+    if (workgroups >= 128 && stages >= 16) {
+      SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
+      launch_big<4, 2, 4, 2, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+                                gated, wblocks, ksplit);
+      SHK_LAUNCH_CHECK("gemm_bf16");
+      return 0;
+    }
+  }
   if (n > 16) {
     // blocks of output rows per workgroup: 8 where that still leaves enough workgroups
     const int mid_waves = (mb >= 4096) ? 8 : 4;

@@ -381,7 +381,8 @@ def test_sample_frequencies_follow_the_distribution(ops):
     "n, m, k",
     [(1, 48, 64), (8, 3584, 3584), (7, 503, 128), (16, 100, 172), (17, 130, 96), (33, 200, 333),
      (48, 64, 64), (64, 1000, 520), (5, 37, 50), (65, 128, 64), (130, 200, 333), (300, 503, 128),
-     (1000, 172, 96), (257, 130, 172), (2048, 1024, 512), (33, 200, 1600), (3, 48, 4000), (64, 100, 2100)],
+     (1000, 172, 96), (257, 130, 172), (2048, 1024, 512), (33, 200, 1600), (3, 48, 4000), (64, 100, 2100),
+     (40, 33000, 1000)],  # the last: 33 to 64 rows on the LDS-staged kernel
 )
 def test_gemm_tiled_weight(ops, n, m, k):
     """The MFMA kernels over the tiled weight layout (weight-streaming up to 64
@@ -525,7 +526,7 @@ def test_attention_mfma_finds_one_far_key_among_thousands(ops):
 
 
 @pytest.mark.parametrize("n, inter, k", [(1, 172, 64), (8, 18944, 256), (20, 100, 96), (40, 352, 128), (64, 48, 50),
-                                         (9, 100, 1700), (50, 64, 3000),
+                                         (9, 100, 1700), (50, 64, 3000), (40, 16400, 1040),
                                          (65, 172, 64), (300, 1000, 520), (1000, 200, 96)])
 def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
     """One product over the interleaved gate/up weight yields silu(x g^T) * (x u^T)."""
@@ -542,7 +543,7 @@ def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
 
 
 @pytest.mark.parametrize("n, m, k", [(8, 3584, 3584), (1, 48, 4000), (33, 200, 1600), (64, 100, 2100),
-                                     (100, 3584, 3584), (300, 136, 1100)])
+                                     (100, 3584, 3584), (300, 136, 1100), (64, 2100, 16400), (40, 2100, 16400)])
 def test_split_product_and_its_readers(ops, n, m, k):
     """A product split along k leaves partial sums; the norm and the cache-write
     kernel add them up in order and give what the unsplit product gives."""
