@@ -70,6 +70,9 @@ class LLMEngine:
         self.eos_ids = set(model.spec.eos_token_ids)
         self.requests: dict[int, Request] = {}
         self.stats = EngineStats()
+        # (batch, prepared step) of the next step, laid out while the device ran the last
+        # one; dropped whenever a request arrives, ends or is aborted
+        self._planned = None
 
     # reference name for the cache manager
     @property
@@ -101,6 +104,7 @@ class LLMEngine:
         req = Request(token_ids=token_ids, sampling=sampling)
         self.requests[req.req_id] = req
         self.scheduler.add(req)
+        self._planned = None
         return req.req_id
 
     @property
@@ -108,7 +112,15 @@ class LLMEngine:
         return self.scheduler.has_work
 
     def step(self) -> list[StepOutput]:
-        batch = self.scheduler.schedule()
+        planned, self._planned = self._planned, None
+        running = self.scheduler.running
+        if planned is not None and (self.scheduler.waiting or len(planned[0]) != len(running)
+                                    or any(p[0] is not r for p, r in zip(planned[0], running))):
+            planned = None  # the queues were changed behind the engine's back
+        if planned is not None:
+            batch, prepared = planned
+        else:
+            batch, prepared = self.scheduler.schedule(), None
         if not batch:
             return []
         entries, sampled = [], []
@@ -121,16 +133,23 @@ class LLMEngine:
             )
             if reaches_end:
                 sampled.append(req)
-        logits = self.runner.step(entries)
-        tokens = self.sampler.sample(logits, sampled)
-        for req, token in zip(sampled, tokens):
-            req.token_ids.append(token)
+        if prepared is not None:
+            logits = self.runner.launch_decode(prepared, [e.tokens[0] for e in entries])
+        else:
+            logits = self.runner.step(entries)
+        chosen = self.sampler.launch(logits, sampled)
 
-        # before finishing: finish() gives the pages back
-        self.scheduler.postprocess(batch)
+        # While the device works: what does not depend on the tokens it will choose.
+        self.scheduler.postprocess(batch)  # before finishing: finish() gives the pages back
+        ahead = self.scheduler.plan_decode_step() if len(sampled) == len(batch) else None
+        if ahead is not None:
+            self._planned = (ahead, self.runner.prepare_decode(
+                [req.cache for req, _ in ahead], [req.num_computed_tokens for req, _ in ahead]))
 
+        tokens = [] if chosen is None else chosen.tolist()  # waits for the device
         outputs: list[StepOutput] = []
         for req, token in zip(sampled, tokens):
+            req.token_ids.append(token)
             self.stats.tokens_generated += 1
             finished, reason = False, None
             if token in self.eos_ids and not req.sampling.ignore_eos:
@@ -141,6 +160,7 @@ class LLMEngine:
             if finished:
                 self.scheduler.finish(req, reason)
                 del self.requests[req.req_id]
+                self._planned = None  # the next step is not the one that was planned
         self.stats.steps += 1
         return outputs
 
@@ -161,6 +181,7 @@ class LLMEngine:
         req = self.requests.pop(req_id, None)
         if req is not None:
             self.scheduler.abort(req)
+            self._planned = None
 
     def metrics(self) -> dict:
         sched, cache = self.scheduler, self.cache

@@ -342,6 +342,38 @@ class ModelRunner:
         host[off["fresh"] : off["fresh"] + n] = 0
         return True
 
+    # ------------------------------------------------------ a step in two halves
+
+    def prepare_decode(self, caches: list, starts: list[int]):
+        """The host's share of a decode step whose tokens are not known yet: one
+        token for each sequence, at position starts[i], logits wanted.  Returns a
+        handle for launch_decode, or None when the step cannot be prepared (no
+        captured graph fits, or its rows changed): step() then does everything."""
+        entries = [StepEntry(c, [0], s, [0]) for c, s in zip(caches, starts)]
+        key = self._graph_key(entries)
+        g = self._graphs.get(key) if key is not None else None
+        if g is None or not self._refresh(g, entries, key[1]):
+            return None
+        return g, entries
+
+    def launch_decode(self, prepared, tokens: list[int]) -> torch.Tensor:
+        """Runs a step that prepare_decode() laid out, now that its tokens are known."""
+        g, entries = prepared
+        n = len(entries)
+        if len(tokens) != n or min(tokens) < 0 or max(tokens) >= self.vocab_size:
+            for e, t in zip(entries, tokens):
+                e.tokens = [t]
+            return self.step(entries)  # raises what an ordinary step raises
+        off = g.offsets["token_ids"]
+        g.host[off : off + n] = tokens
+        g.meta_dev.copy_(g.pinned, non_blocking=True)
+        g.copied.record()
+        g.graph.replay()
+        self.graph_replays += 1
+        for e in entries:
+            e.cache.fresh_state = False
+        return g.logits[:n]
+
     # -------------------------------------------------------------------- step
 
     def step(self, entries: list[StepEntry]) -> torch.Tensor:

@@ -111,6 +111,30 @@ class Scheduler:
 
         return singles + portions
 
+    def plan_decode_step(self) -> list[tuple[Request, int]] | None:
+        """What the next schedule() will return if every running request goes on
+        with the one token that is being sampled for it right now and nothing
+        arrives meanwhile: that token for each of them, in admission order.  Called
+        after postprocess() and before the sampled tokens are known, so that the
+        host prepares the next step while the device still computes this one.
+        None when the next step is not of this kind (somebody waits, a prompt is
+        in progress, a request reaches its length, the budget or the pages do not
+        suffice): schedule() then decides as ever.  Pages taken here are those
+        schedule() would take; a request that ends after all gives them back with
+        the rest."""
+        if self.waiting or not self.running or len(self.running) > self.max_tokens_per_step:
+            return None
+        for req in self.running:
+            if req.status is not Status.RUNNING or req.num_computed_tokens != req.num_tokens:
+                return None
+            if req.num_generated + 1 >= req.sampling.max_new_tokens:
+                return None
+        for req in self.running:
+            if not self.cache.can_append(req.cache, req.num_computed_tokens, 1):
+                return None  # schedule() finds the same shortage, and preempts
+            self.cache.append(req.cache, req.num_computed_tokens, 1)
+        return [(req, 1) for req in self.running]
+
     def postprocess(self, batch: list[tuple[Request, int]]) -> None:
         """Count the step's tokens as computed, publish full pages for prefix
         sharing, and give back pages that a window has passed."""

@@ -40,15 +40,17 @@ class Sampler:
             return req.sampling.seed
         return splitmix64((self.engine_seed << 20) ^ req.req_id)
 
-    def sample(self, logits: torch.Tensor, reqs: list) -> list[int]:
-        """logits float32 [R, vocab] on the device, one row per request."""
+    def launch(self, logits: torch.Tensor, reqs: list) -> torch.Tensor | None:
+        """Starts the choice of one token per row of logits (float32 [R, vocab]
+        on the device, one row per request) and returns the device tensor that
+        will hold them; nothing here waits for the device."""
         if not reqs:
-            return []
+            return None
         rows, vocab = logits.shape
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
         if all(r.sampling.temperature == 0.0 for r in reqs):
             ops.argmax(logits, out)
-            return out.tolist()
+            return out
         params = torch.tensor(
             [[r.sampling.temperature for r in reqs],
              [r.sampling.top_p for r in reqs],
@@ -58,4 +60,9 @@ class Sampler:
         if self._scratch is None or self._scratch.numel() < rows * vocab:
             self._scratch = torch.empty(rows * vocab, dtype=torch.float32, device=logits.device)
         ops.sample(logits, out, params[0], params[1], params[2], self._scratch)
-        return out.tolist()
+        return out
+
+    def sample(self, logits: torch.Tensor, reqs: list) -> list[int]:
+        """The tokens themselves: launch(), then the wait for the device."""
+        out = self.launch(logits, reqs)
+        return [] if out is None else out.tolist()

@@ -213,3 +213,51 @@ def test_random_workloads_keep_the_invariants(seed):
                     finished += 1
         cm.check([r.cache for r in sched.running])
     assert finished == 12 and cm.num_free == 10 and cm.slots.num_free == 16
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_a_planned_decode_step_is_the_step_that_schedule_would_give(seed):
+    """Two schedulers get the same requests, arrivals and tokens.  One plans its
+    next step ahead whenever plan_decode_step() offers one (before the step's
+    tokens exist); the other always calls schedule().  Their batches and their
+    pools agree at every step, through admissions, ends and preemptions."""
+    rng = random.Random(seed)
+    cms = [cache(9, 4), cache(9, 4)]
+    scheds = [Scheduler(cm, max_tokens_per_step=10, max_running=4) for cm in cms]
+    arrivals = sorted((rng.randrange(60), [rng.randrange(50) for _ in range(rng.randint(1, 9))],
+                       rng.randint(1, 12)) for _ in range(10))
+    reqs = [{}, {}]  # arrival number -> request, per scheduler
+    planned, steps, plans_used = None, 0, 0
+    while arrivals or any(s.has_work for s in scheds):
+        steps += 1
+        assert steps < 3000
+        while arrivals and arrivals[0][0] <= steps:
+            _, tokens, max_new = arrivals.pop(0)
+            for which in (0, 1):
+                r = req(tokens, max_new)
+                reqs[which][len(reqs[which])] = r
+                scheds[which].add(r)
+            planned = None  # as the engine does when a request arrives
+        if planned is not None:
+            plans_used += 1
+        batches = [planned if planned is not None else scheds[0].schedule(), scheds[1].schedule()]
+        number = [{r.req_id: k for k, r in reqs[w].items()} for w in (0, 1)]
+        assert [(number[0][r.req_id], n) for r, n in batches[0]] == \
+               [(number[1][r.req_id], n) for r, n in batches[1]]
+        assert cms[0].num_free == cms[1].num_free
+        for w in (0, 1):
+            scheds[w].postprocess(batches[w])
+        ends = [r.num_computed_tokens == r.num_tokens for r, _ in batches[0]]
+        planned = scheds[0].plan_decode_step() if all(ends) and batches[0] else None
+        token = rng.randrange(50)
+        for w in (0, 1):
+            for (r, _), end in zip(list(batches[w]), ends):
+                if end:
+                    r.token_ids.append(token)
+                    if r.num_generated >= r.sampling.max_new_tokens:
+                        scheds[w].finish(r, "length")
+                        if w == 0:
+                            planned = None
+            cms[w].check([r.cache for r in scheds[w].running])
+    assert plans_used > 5
+    assert all(cm.num_free == 9 for cm in cms)
