@@ -451,9 +451,16 @@ __global__ void __launch_bounds__(GM* GN* kWave)
   // blocks of 32 (up to 8 token tiles of 32 / that many weight tiles) and block B goes to
   // die B % 8, whose 32 compute units then work on tiles that share their
   // operands: the die's L2 serves most of their loads.
-  // With too few tiles for that (by_die == 0) they are taken in plain order.
+  // With fewer tiles (by_die == 2 * dx) the grid of tiles is cut into dx x 8/dx
+  // rectangles, one for each die, where the numbers of tiles allow that; else
+  // (by_die == 0) the tiles are taken in plain order.
   int tile_x = blockIdx.x % tiles_x, tile_y = blockIdx.x / tiles_x;
-  if (by_die) {
+  if (by_die > 1) {
+    const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
+    const int dx = by_die / 2, wide = tiles_x / dx, high = tiles_y / (kDies / dx);
+    tile_x = (die % dx) * wide + turn % wide;
+    tile_y = (die / dx) * high + turn / wide;
+  } else if (by_die) {
     const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
     const int block_y = tiles_y < 8 ? tiles_y : 8, block_x = kDieUnits / block_y;
     const int blocks_x = (tiles_x + block_x - 1) / block_x;
@@ -727,8 +734,20 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
   const long long blocks = static_cast<long long>((tiles_x + block_x - 1) / block_x) *
                            ((tiles_y + block_y - 1) / block_y);
   // worth it from four rounds of workgroups on: below that, whole dies would stay idle
-  const int by_die = static_cast<long long>(tiles_x) * tiles_y >= 4 * kDies * kDieUnits;
-  dim3 grid(by_die ? static_cast<unsigned>((blocks + kDies - 1) / kDies * kDies * kDieUnits)
+  int by_die = static_cast<long long>(tiles_x) * tiles_y >= 4 * kDies * kDieUnits;
+  if (!by_die) {
+    // one rectangle of tiles per die, cut so that a die's tiles share the most
+    // operands (the fewest rows of weights and activations to read per die)
+    long long least = 0;
+    for (int dx = 1; dx <= kDies; dx *= 2) {
+      const int dy = kDies / dx;
+      if (tiles_x % dx || tiles_y % dy) continue;
+      const long long rows = static_cast<long long>(tiles_x / dx) * (16 * GM * WM) +
+                             static_cast<long long>(tiles_y / dy) * (16 * GN * WN);
+      if (!least || rows < least) least = rows, by_die = 2 * dx;
+    }
+  }
+  dim3 grid(by_die == 1 ? static_cast<unsigned>((blocks + kDies - 1) / kDies * kDies * kDieUnits)
                    : static_cast<unsigned>(tiles_x * tiles_y),
             ksplit);
   if (gated) {
