@@ -12,6 +12,8 @@
 // wavefronts per block of 16 weight rows; the wavefronts take the k-tiles
 // round-robin and their partial sums are added in a fixed order through LDS.
 // The weights are read exactly once from HBM; accumulation is float32.
+#include <cstdlib>
+
 #include "api.h"
 #include "common.h"
 
@@ -417,6 +419,54 @@ __global__ void __launch_bounds__(WAVES* kWave)
   }
 }
 
+// What a wavefront of the large kernels does with its WM x WN accumulator tiles:
+// lane (j, kg) of tile (i, jn) holds token tok_first + jn*16 + j, rows
+// (block_first + i)*16 + kg*4 + r.  Gated: weight blocks come in (gate, up) pairs
+// that make one block of output rows.  share: which float32 partial sum [share][n][m].
+template <int WM, int WN, bool GATED>
+__device__ __forceinline__ void big_store(const f32x4 (&acc)[WM][WN], int lane, int tok_first,
+                                          int block_first, int n, int m,
+                                          const float* __restrict__ bias, void* __restrict__ out,
+                                          int ldo, int out_f32, int accumulate, int share) {
+  const int j = lane % 16, kg = lane / 16;
+#pragma unroll
+  for (int jn = 0; jn < WN; ++jn) {
+    const int token = tok_first + jn * 16 + j;
+    if (token >= n) continue;
+#pragma unroll
+    for (int i = 0; i < WM; i += (GATED ? 2 : 1)) {
+      // gated: weight blocks come in (gate, up) pairs that make one block of output rows
+      const int row0 = (GATED ? (block_first + i) / 2 : block_first + i) * 16 + kg * 4;
+      if (row0 >= m) continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r] : acc[i][jn][r];
+        if (bias && row0 + r < m) v[r] += bias[row0 + r];
+      }
+      const size_t idx = (static_cast<size_t>(share) * n + token) * ldo + row0;
+      if (out_f32) {
+        float* o = static_cast<float*>(out) + idx;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+      } else {
+        bf16* o = static_cast<bf16*>(out) + idx;
+        if (row0 + 3 < m && (ldo & 3) == 0) {
+          uint2 packed;
+          packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+          packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+          *reinterpret_cast<uint2*>(o) = packed;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (row0 + r < m) o[r] = from_float<bf16>(v[r]);
+        }
+      }
+    }
+  }
+}
+
 // gemm_big_kernel: for many tokens (prompt portions).  A workgroup of 4 or 8
 // wavefronts computes a tile of weight rows x tokens, each wavefront a part of
 // it as WM x WN MFMA tiles.  Per stage of k, the weights' tiles (already in
@@ -428,6 +478,34 @@ __global__ void __launch_bounds__(WAVES* kWave)
 
 constexpr int kDies = 8;        // accelerator dies (XCDs), each with an L2 of its own
 constexpr int kDieUnits = 32;  // compute units per die
+
+// The tile of a workgroup of the large kernels; false: none (the grid is padded).
+__device__ __forceinline__ bool big_tile(int tiles_x, int tiles_y, int by_die, int& tile_x, int& tile_y) {
+  // Which tile: workgroups are handed to the chip's eight dies (each with its own
+  // L2) in turn, workgroup p to die p % 8.  The tiles are therefore dealt out in
+  // blocks of 32 (up to 8 token tiles of 32 / that many weight tiles) and block B goes to
+  // die B % 8, whose 32 compute units then work on tiles that share their
+  // operands: the die's L2 serves most of their loads.
+  // With fewer tiles (by_die == 2 * dx) the grid of tiles is cut into dx x 8/dx
+  // rectangles, one for each die, where the numbers of tiles allow that; else
+  // (by_die == 0) the tiles are taken in plain order.
+  tile_x = blockIdx.x % tiles_x, tile_y = blockIdx.x / tiles_x;
+  if (by_die > 1) {
+    const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
+    const int dx = by_die / 2, wide = tiles_x / dx, high = tiles_y / (kDies / dx);
+    tile_x = (die % dx) * wide + turn % wide;
+    tile_y = (die / dx) * high + turn / wide;
+  } else if (by_die) {
+    const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
+    const int block_y = tiles_y < 8 ? tiles_y : 8, block_x = kDieUnits / block_y;
+    const int blocks_x = (tiles_x + block_x - 1) / block_x;
+    const int block = (turn / kDieUnits) * kDies + die, within = turn % kDieUnits;
+    tile_x = (block % blocks_x) * block_x + within / block_y;
+    tile_y = (block / blocks_x) * block_y + within % block_y;
+    if (within >= block_x * block_y) return false;
+  }
+  return tile_x < tiles_x && tile_y < tiles_y;
+}
 
 // GM x GN wavefronts per workgroup, each with WM x WN MFMA tiles (16 x 16): the
 // workgroup covers 16*GM*WM weight rows x 16*GN*WN tokens.  KS: MFMA steps (32 of
@@ -446,30 +524,8 @@ __global__ void __launch_bounds__(GM* GN* kWave)
   auto stage = [&](int buf, int frag) -> uint4* { return stage_mem + (buf * kFrags + frag) * kWave; };
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int wm = wave / GN, wn = wave % GN;  // place of the wavefront in the workgroup's tile
-  // Which tile: workgroups are handed to the chip's eight dies (each with its own
-  // L2) in turn, workgroup p to die p % 8.  The tiles are therefore dealt out in
-  // blocks of 32 (up to 8 token tiles of 32 / that many weight tiles) and block B goes to
-  // die B % 8, whose 32 compute units then work on tiles that share their
-  // operands: the die's L2 serves most of their loads.
-  // With fewer tiles (by_die == 2 * dx) the grid of tiles is cut into dx x 8/dx
-  // rectangles, one for each die, where the numbers of tiles allow that; else
-  // (by_die == 0) the tiles are taken in plain order.
-  int tile_x = blockIdx.x % tiles_x, tile_y = blockIdx.x / tiles_x;
-  if (by_die > 1) {
-    const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
-    const int dx = by_die / 2, wide = tiles_x / dx, high = tiles_y / (kDies / dx);
-    tile_x = (die % dx) * wide + turn % wide;
-    tile_y = (die / dx) * high + turn / wide;
-  } else if (by_die) {
-    const int die = blockIdx.x % kDies, turn = blockIdx.x / kDies;
-    const int block_y = tiles_y < 8 ? tiles_y : 8, block_x = kDieUnits / block_y;
-    const int blocks_x = (tiles_x + block_x - 1) / block_x;
-    const int block = (turn / kDieUnits) * kDies + die, within = turn % kDieUnits;
-    tile_x = (block % blocks_x) * block_x + within / block_y;
-    tile_y = (block / blocks_x) * block_y + within % block_y;
-    if (within >= block_x * block_y) return;
-  }
-  if (tile_x >= tiles_x || tile_y >= tiles_y) return;
+  int tile_x, tile_y;
+  if (!big_tile(tiles_x, tiles_y, by_die, tile_x, tile_y)) return;
   const int mb0 = tile_x * (GM * WM);  // first block of 16 weight rows
   const int tok0 = tile_y * (16 * GN * WN);
   // blocks of 16 weight rows; a gated weight has two per 16 output rows
@@ -624,45 +680,155 @@ __global__ void __launch_bounds__(GM* GN* kWave)
     }
   }
 
-  // lane (j, kg) of tile (i, jn): token tok0 + (wn*WN + jn)*16 + j,
-  // rows (mb0 + wm*WM + i)*16 + kg*4 + r
-  const int j = lane % 16, kg = lane / 16;
+  big_store<WM, WN, GATED>(acc, lane, tok0 + wn * WN * 16, mb0 + wm * WM, n, m, bias, out, ldo, out_f32,
+                           accumulate, blockIdx.y);
+}
+
+// gemm_big_lds_kernel: the same tiles, for aligned activations and whole stages
+// of k, with the operands loaded from global memory straight into LDS
+// (global_load_lds_dwordx4: lane l's 16 bytes land at l * 16 of the fragment, the
+// layout above) instead of through registers.  Four stage buffers (three for the
+// largest stages); the loads of the next two stages (one) are in flight while a
+// stage is multiplied, and one barrier
+// per stage both publishes a stage and frees the buffer of the stage before.
+// The compiler cannot see when another wavefront's load has landed: every
+// wavefront waits for its own loads of the stage (s_waitcnt vmcnt, counting the
+// loads issued since) before the barrier.  Each buffer is an LDS array of its
+// own, so that the compiler's own bookkeeping tells the buffers apart and adds
+// no wait for loads into another one.
+#define SHK_LOAD_TO_LDS(gptr, lptr)                                                        \
+  __builtin_amdgcn_global_load_lds(                                                       \
+      reinterpret_cast<const __attribute__((address_space(1))) void*>(                    \
+          reinterpret_cast<uintptr_t>(gptr)),                                             \
+      (__attribute__((address_space(3))) void*)(lptr), 16, 0, 0)
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maxima)
+#define SHK_WAIT_LOADS(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
+
+template <int GM, int GN, int WM, int WN, int KS, bool GATED>
+__global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per_eu(2)))
+    gemm_big_lds_kernel(const bf16* __restrict__ a, int lda, int n, int k,
+                        const uint4* __restrict__ wt, int ktiles, int m,
+                        const float* __restrict__ bias, void* __restrict__ out, int ldo,
+                        int out_f32, int accumulate, int ksplit, int tiles_x, int tiles_y,
+                        int by_die) {
+  constexpr int kWaves = GM * GN;
+  constexpr int kWFrags = GM * WM * KS, kAFrags = GN * WN * KS, kFrags = kWFrags + kAFrags;
+  constexpr int kWPer = kWFrags / kWaves, kAPer = kAFrags / kWaves;
+  constexpr int kLoads = kWPer + kAPer;  // per wavefront and stage
+  static_assert(kWFrags % kWaves == 0 && kAFrags % kWaves == 0, "fragments must divide among the wavefronts");
+  // four stage buffers where they fit into the 160 KiB of LDS, else three
+  constexpr int NS = 4 * kFrags * kWave * 16 <= 160 * 1024 ? 4 : 3;
+  static_assert(NS * kFrags * kWave * 16 <= 160 * 1024, "three stages must fit in LDS");
+  __shared__ u32x4 stage0[kFrags][kWave], stage1[kFrags][kWave], stage2[kFrags][kWave],
+      stage3[NS == 4 ? kFrags : 1][kWave];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int wm = wave / GN, wn = wave % GN;
+  int tile_x, tile_y;
+  if (!big_tile(tiles_x, tiles_y, by_die, tile_x, tile_y)) return;
+  const int mb0 = tile_x * (GM * WM);
+  const int tok0 = tile_y * (16 * GN * WN);
+  const int mblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
+  const int all_stages = ktiles / KS;  // the host sends only whole stages here
+  const int per_split = (all_stages + ksplit - 1) / ksplit;
+  const int st_first = blockIdx.y * per_split;
+  const int nstages = st_first + per_split < all_stages ? st_first + per_split : all_stages;
+
+  f32x4 acc[WM][WN];
 #pragma unroll
-  for (int jn = 0; jn < WN; ++jn) {
-    const int token = tok0 + (wn * WN + jn) * 16 + j;
-    if (token >= n) continue;
+  for (int i = 0; i < WM; ++i)
 #pragma unroll
-    for (int i = 0; i < WM; i += (GATED ? 2 : 1)) {
-      // gated: weight blocks come in (gate, up) pairs that make one block of output rows
-      const int row0 = (GATED ? (mb0 + wm * WM + i) / 2 : mb0 + wm * WM + i) * 16 + kg * 4;
-      if (row0 >= m) continue;
-      float v[4];
+    for (int jn = 0; jn < WN; ++jn) acc[i][jn] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // what this wavefront loads: fragments wave, wave + kWaves, ... of either operand,
+  // from rows clamped into the matrices (their products are never stored)
+  const uint4* wsrc[kWPer];
+  const bf16* asrc[kAPer];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r] : acc[i][jn][r];
-        if (bias && row0 + r < m) v[r] += bias[row0 + r];
-      }
-      const size_t idx = (static_cast<size_t>(blockIdx.y) * n + token) * ldo + row0;
-      if (out_f32) {
-        float* o = static_cast<float*>(out) + idx;
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
-      } else {
-        bf16* o = static_cast<bf16*>(out) + idx;
-        if (row0 + 3 < m && (ldo & 3) == 0) {
-          uint2 packed;
-          packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
-          packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
-          *reinterpret_cast<uint2*>(o) = packed;
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (row0 + r < m) o[r] = from_float<bf16>(v[r]);
-        }
-      }
-    }
+  for (int i = 0; i < kWPer; ++i) {
+    const int rb = (wave + kWaves * i) / KS;
+    const int block = mb0 + rb < mblocks ? mb0 + rb : mblocks - 1;
+    wsrc[i] = wt + static_cast<size_t>(block) * ktiles * kWave + lane;
   }
+#pragma unroll
+  for (int i = 0; i < kAPer; ++i) {
+    const int rb = (wave + kWaves * i) / KS;
+    const int token = tok0 + rb * 16 + lane % 16;
+    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (lane / 16) * 8;
+  }
+  auto load = [&](u32x4 (&buf)[kFrags][kWave], int st) {
+    const int stage = st < all_stages ? st : 0;  // past the end: any stage, never multiplied
+#pragma unroll
+    for (int i = 0; i < kAPer; ++i) {
+      const int col = (stage * KS + (wave + kWaves * i) % KS) * 32;  // + (lane / 16) * 8 in asrc
+      SHK_LOAD_TO_LDS(asrc[i] + (col + (lane / 16) * 8 < k ? col : 0), &buf[kWFrags + wave + kWaves * i][0]);
+    }
+#pragma unroll
+    for (int i = 0; i < kWPer; ++i) {
+      const int kt = stage * KS + (wave + kWaves * i) % KS;
+      SHK_LOAD_TO_LDS(wsrc[i] + static_cast<size_t>(kt) * kWave, &buf[wave + kWaves * i][0]);
+    }
+  };
+  auto multiply = [&](const u32x4 (&buf)[kFrags][kWave]) {
+    u32x4 af[KS][WN], wf[KS][WM];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+      for (int jn = 0; jn < WN; ++jn) af[ks][jn] = buf[kWFrags + (wn * WN + jn) * KS + ks][lane];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) wf[ks][i] = buf[(wm * WM + i) * KS + ks][lane];
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int jn = 0; jn < WN; ++jn)
+          acc[i][jn] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, wf[ks][i]), __builtin_bit_cast(bf16x8, af[ks][jn]),
+              acc[i][jn], 0, 0, 0);
+  };
+  // The stage in `now` has landed for every wavefront once each has waited for its
+  // own loads (the younger stages may stay in flight) and met the others; after the
+  // barrier nobody reads the stage before any more, so its buffer takes new loads.
+#define SHK_LDS_STEP(now, refill, st_refill)  \
+  SHK_WAIT_LOADS((NS - 2) * kLoads);          \
+  asm volatile("" ::: "memory");              \
+  __builtin_amdgcn_s_barrier();               \
+  asm volatile("" ::: "memory");              \
+  load(refill, st_refill);                    \
+  __builtin_amdgcn_sched_barrier(0);          \
+  multiply(now);
+  int st = st_first;
+  if constexpr (NS == 4) {
+    load(stage0, st_first);
+    load(stage1, st_first + 1);
+    load(stage2, st_first + 2);
+    for (; st + 3 < nstages; st += 4) {
+      SHK_LDS_STEP(stage0, stage3, st + 3)
+      SHK_LDS_STEP(stage1, stage0, st + 4)
+      SHK_LDS_STEP(stage2, stage1, st + 5)
+      SHK_LDS_STEP(stage3, stage2, st + 6)
+    }
+    if (st < nstages) { SHK_LDS_STEP(stage0, stage3, st + 3) }
+    if (st + 1 < nstages) { SHK_LDS_STEP(stage1, stage0, st + 4) }
+    if (st + 2 < nstages) { SHK_LDS_STEP(stage2, stage1, st + 5) }
+  } else {
+    load(stage0, st_first);
+    load(stage1, st_first + 1);
+    for (; st + 2 < nstages; st += 3) {
+      SHK_LDS_STEP(stage0, stage2, st + 2)
+      SHK_LDS_STEP(stage1, stage0, st + 3)
+      SHK_LDS_STEP(stage2, stage1, st + 4)
+    }
+    if (st < nstages) { SHK_LDS_STEP(stage0, stage2, st + 2) }
+    if (st + 1 < nstages) { SHK_LDS_STEP(stage1, stage0, st + 3) }
+  }
+#undef SHK_LDS_STEP
+  SHK_WAIT_LOADS(0);  // no load may arrive in LDS that the workgroup has given back
+
+  big_store<WM, WN, GATED>(acc, lane, tok0 + wn * WN * 16, mb0 + wm * WM, n, m, bias, out, ldo, out_f32,
+                           accumulate, blockIdx.y);
 }
 
 }  // namespace shk
@@ -750,6 +916,24 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
   dim3 grid(by_die == 1 ? static_cast<unsigned>((blocks + kDies - 1) / kDies * kDies * kDieUnits)
                    : static_cast<unsigned>(tiles_x * tiles_y),
             ksplit);
+  // The kernel that loads straight into LDS, for workgroups that have a compute unit
+  // to themselves anyway (its three or four stage buffers leave no room for a
+  // second) and at least 128 tokens (with 64 it measured 3 % slower).
+  if constexpr (GM * GN >= 8 && GN * WN >= 8 &&
+                3 * (GM * WM + GN * WN) * KS * kWave * 16 <= 160 * 1024) {
+    // (SHK_NO_LDS_LOADS=1 in the environment keeps to the kernel that stages through
+    // registers: for comparing the two)
+    static const bool direct = getenv("SHK_NO_LDS_LOADS") == nullptr;
+    if (direct && vec && kt % KS == 0) {
+      if (gated)
+        gemm_big_lds_kernel<GM, GN, WM, WN, KS, true><<<grid, GM * GN * kWave, 0, s>>>(
+            ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, ksplit, tiles_x, tiles_y, by_die);
+      else
+        gemm_big_lds_kernel<GM, GN, WM, WN, KS, false><<<grid, GM * GN * kWave, 0, s>>>(
+            ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, ksplit, tiles_x, tiles_y, by_die);
+      return;
+    }
+  }
   if (gated) {
     auto kernel = gemm_big_kernel<GM, GN, WM, WN, KS, true>;
     if (lds > 65536)

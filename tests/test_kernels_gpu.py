@@ -408,6 +408,41 @@ def test_gemm_tiled_weight(ops, n, m, k):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize(
+    "n, m, k, gated",
+    [(1000, 16384, 288, False),  # tiles of 256 x 256, the last token tile partly empty
+     (2048, 3584, 192, False),   # tiles of 256 x 128, stages of 64: three of them
+     (2000, 3600, 448, False),   # the same with a partly empty tile on both sides, seven stages
+     (1000, 8192, 352, True)],   # gated, 256 x 256, eleven stages
+)
+def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
+    """The large tiles with aligned rows and whole stages of k: operands go from
+    global memory into LDS without passing through registers; every count of
+    stages ends the ring of stage buffers at another place."""
+    torch.manual_seed(21)
+    dtype = torch.bfloat16
+    a = torch.randn(n, k)
+    if gated:
+        g, u = torch.randn(m, k) / math.sqrt(k) * 2, torch.randn(m, k) / math.sqrt(k)
+        wt = ops.interleave_gate_up(dev(g, dtype), dev(u, dtype))
+        gate = rounded(a, dtype) @ rounded(g, dtype).t()
+        want = gate * torch.sigmoid(gate) * (rounded(a, dtype) @ rounded(u, dtype).t())
+        out = torch.full((n, m), float("nan"), device="cuda", dtype=dtype)
+        ops.gemm_tiled_weight(dev(a, dtype), wt, m, k, out, gated=True)
+        close(out, want, dtype)
+        return
+    w, b = torch.randn(m, k) / math.sqrt(k), torch.randn(m)
+    want = rounded(a, dtype) @ rounded(w, dtype).t() + b.double()
+    wt = ops.retile_weight(dev(w, dtype))
+    out = torch.full((n, m), float("nan"), device="cuda", dtype=dtype)
+    ops.gemm_tiled_weight(dev(a, dtype), wt, m, k, out, bias=dev(b))
+    close(out, want, dtype)
+    # a row's result does not depend on the rows around it
+    part = torch.empty(300, m, device="cuda", dtype=dtype)
+    ops.gemm_tiled_weight(dev(a, dtype)[500:800], wt, m, k, part, bias=dev(b))
+    assert torch.equal(part, out[500:800])
+
+
 def test_gemm_tiled_weight_rows_do_not_depend_on_the_rest_of_the_batch(ops):
     """Within one kernel (up to 16 rows, 17 to 64, more) a row's result is bit
     for bit the same whatever else is in the call; between kernels the order of
