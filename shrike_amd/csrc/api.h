@@ -118,15 +118,18 @@ int shk_attention_prefill_bf16(const void* q, int q_stride, void* out, int num_t
 // The same for all query heads of a key/value head at once: a workgroup serves
 // `tiles` = shk_attention_prefill_shared_tiles(...) consecutive 16-query tiles of
 // one sequence (wg_seq, wg_q0 in steps of 16 * tiles) and stages each chunk of
-// keys once in LDS.  tiles == 0: the shape is not served (more than 8 query
-// heads per key/value head, head_dim > 128).
-int shk_attention_prefill_shared_tiles(int heads, int kv_heads, int head_dim);
+// keys once in LDS.  small != 0: workgroups of 8 wavefronts instead of 16, with
+// half as many tiles each, for portions that would otherwise make too few
+// workgroups for the chip.  tiles == 0: the shape is not served (more query
+// heads per key/value head than a workgroup has wavefronts, head_dim > 128).
+int shk_attention_prefill_shared_tiles(int heads, int kv_heads, int head_dim, int small);
 int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out, int num_wgs,
                                       int heads, int kv_heads, int head_dim, const int32_t* cu_q,
                                       const int32_t* ctx_lens, const int32_t* wg_seq,
                                       const int32_t* wg_q0, const int32_t* tables,
                                       int table_stride, const void* k_pool, const void* v_pool,
-                                      int page_size, int window, float scale, void* stream);
+                                      int page_size, int window, float scale, int small,
+                                      void* stream);
 
 // out[r] = lowest index of the largest value of logits[r, :vocab].  Rows wider
 // than 4096 are searched in chunks; scratch then holds

@@ -686,11 +686,12 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
 // in steps of 16 * tiles queries.
 
 constexpr int kUnitsPerWave = 1;
-constexpr int kSharedWaves = 16;
+// wavefronts per workgroup: 16, or 8 where that many would make too few workgroups
+// for the chip (a portion of a few hundred queries)
+constexpr int kSharedWaves = 16, kSharedWavesSmall = 8;
 
-template <int D>
-__global__ void __launch_bounds__(kSharedWaves* kWave)
-    __attribute__((amdgpu_waves_per_eu(kSharedWaves >= 16 ? 4 : 2)))
+template <int D, int WAVES>
+__global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_eu(4)))
     attention_prefill_shared_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                                     int heads, int kv_heads, int tiles,
                                     const int32_t* __restrict__ cu_q,
@@ -703,7 +704,7 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
   constexpr int U = kUnitsPerWave;
   constexpr int kKFrags = 2 * (D / 32), kVFrags = D / 16, kFrags = kKFrags + kVFrags;
   // fragments each wavefront stages; where they do not divide, some are staged twice
-  constexpr int kPer = (kFrags + kSharedWaves - 1) / kSharedWaves;
+  constexpr int kPer = (kFrags + WAVES - 1) / WAVES;
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
   __shared__ u32x4 kv[2][kFrags][kWave];
 
@@ -756,7 +757,7 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
     for (int db = 0; db < D / 16; ++db) o[u][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- staging.  Wavefront w fetches fragments w, w + kSharedWaves, ...  Fragment f < kKFrags
+  // ---- staging.  Wavefront w fetches fragments w, w + WAVES, ...  Fragment f < kKFrags
   // is K tile f / (D/32), head_dim slice f % (D/32); row i of K tile t is key
   // 8*(i/4) + 4*t + i%4 of the chunk, so that lane (j, g) of a score tile ends up
   // with the eight keys 8*g .. 8*g + 7.  The others are V^T blocks of 16 elements.
@@ -766,7 +767,7 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
   bool is_k[kPer];
 #pragma unroll
   for (int i = 0; i < kPer; ++i) {
-    const int f = (wave + kSharedWaves * i) % kFrags;
+    const int f = (wave + WAVES * i) % kFrags;
     is_k[i] = f < kKFrags;
     if (is_k[i]) {
       const int t = f / (D / 32), ds = f % (D / 32);
@@ -811,7 +812,7 @@ __global__ void __launch_bounds__(kSharedWaves* kWave)
         }
         x &= keep;
       }
-      kv[buf][(wave + kSharedWaves * i) % kFrags][lane] = x;
+      kv[buf][(wave + WAVES * i) % kFrags][lane] = x;
     }
   };
 
@@ -957,11 +958,16 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
                                   const int32_t* ctx_lens, const int32_t* wg_seq,
                                   const int32_t* wg_q0, const int32_t* tables, int table_stride,
                                   const bf16* k_pool, const bf16* v_pool, int page_size, int window,
-                                  float scale) {
+                                  float scale, bool small) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
-  attention_prefill_shared_kernel<D><<<grid, kSharedWaves * kWave, 0, s>>>(
-      q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables, table_stride,
-      k_pool, v_pool, page_size, magic, window, scale);
+  if (small)
+    attention_prefill_shared_kernel<D, kSharedWavesSmall><<<grid, kSharedWavesSmall * kWave, 0, s>>>(
+        q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
+        table_stride, k_pool, v_pool, page_size, magic, window, scale);
+  else
+    attention_prefill_shared_kernel<D, kSharedWaves><<<grid, kSharedWaves * kWave, 0, s>>>(
+        q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
+        table_stride, k_pool, v_pool, page_size, magic, window, scale);
 }
 
 }  // namespace shk
@@ -1034,10 +1040,11 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
 
 // Query tiles of 16 that one workgroup of the shared-key prefill kernel serves for
 // a given number of query heads per key/value head; 0: the shape is not served.
-extern "C" int shk_attention_prefill_shared_tiles(int heads, int kv_heads, int head_dim) {
+extern "C" int shk_attention_prefill_shared_tiles(int heads, int kv_heads, int head_dim, int small) {
   const int group = heads / kv_heads;
-  if (group < 1 || group > kUnitsPerWave * kSharedWaves || head_dim > 128) return 0;
-  return (kUnitsPerWave * kSharedWaves) / group;
+  const int units = kUnitsPerWave * (small ? kSharedWavesSmall : kSharedWaves);
+  if (group < 1 || group > units || head_dim > 128) return 0;
+  return units / group;
 }
 
 extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out,
@@ -1047,10 +1054,10 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
                                                  const int32_t* wg_q0, const int32_t* tables,
                                                  int table_stride, const void* k_pool,
                                                  const void* v_pool, int page_size, int window,
-                                                 float scale, void* stream) {
+                                                 float scale, int small, void* stream) {
   if (check_mfma_shapes("attention_prefill_shared", heads, kv_heads, head_dim, page_size, q_stride))
     return 1;
-  const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim);
+  const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim, small);
   SHK_REQUIRE(tiles > 0, "attention_prefill_shared: %d query heads per key/value head or head_dim %d "
               "is not served", heads / kv_heads, head_dim);
   SHK_REQUIRE(num_wgs >= 0 && kv_heads <= 65535, "attention_prefill_shared: bad sizes");
@@ -1069,7 +1076,7 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
   launch_prefill_shared<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
                            heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,      \
                            table_stride, static_cast<const bf16*>(k_pool),                     \
-                           static_cast<const bf16*>(v_pool), page_size, window, scale)
+                           static_cast<const bf16*>(v_pool), page_size, window, scale, small != 0)
   switch (head_dim) {
     case 32: CALL(32); break;
     case 64: CALL(64); break;

@@ -99,10 +99,16 @@ class Runtime:
                                      spec.scale, partial, nsplit)
             tiles = ops.attention_prefill_shared_tiles(h, hkv, d) if ctx.num_prefill_tiles else 0
             if tiles:
+                # few queries: smaller workgroups, so that there are enough for the chip
+                small = -(-ctx.num_prefill_tiles // tiles) * hkv < PREFILL_MIN_WORKGROUPS
+                if small and ops.attention_prefill_shared_tiles(h, hkv, d, small=True):
+                    tiles = ops.attention_prefill_shared_tiles(h, hkv, d, small=True)
+                else:
+                    small = False
                 wg_seq, wg_q0, count = ctx.prefill_workgroups(tiles)
                 ops.attention_prefill_shared(q, out, count, h, hkv, d, ctx.cu_q, ctx.ctx_lens, wg_seq,
                                              wg_q0, tables, cache.k_pool, cache.v_pool,
-                                             cache.page_size, spec.window, spec.scale)
+                                             cache.page_size, spec.window, spec.scale, small=small)
             elif ctx.num_prefill_tiles:
                 ops.attention_prefill(q, out, ctx.num_prefill_tiles, h, hkv, d, ctx.cu_q,
                                       ctx.ctx_lens, ctx.tile_seq, ctx.tile_q0, tables, cache.k_pool,
@@ -110,6 +116,10 @@ class Runtime:
             return
         ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.k_pool,
                       cache.v_pool, cache.page_size, spec.window, spec.scale)
+
+
+# portions whose 16-wavefront workgroups would number fewer than this take 8-wavefront ones
+PREFILL_MIN_WORKGROUPS = 192
 
 
 def bucket(n: int, floor: int = 1) -> int:

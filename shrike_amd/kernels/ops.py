@@ -335,15 +335,17 @@ def attention_prefill(q, out, num_tiles, heads, kv_heads, head_dim, cu_q, ctx_le
     )
 
 
-def attention_prefill_shared_tiles(heads, kv_heads, head_dim) -> int:
-    """16-query tiles per workgroup of attention_prefill_shared; 0 if the shape is not served."""
-    return int(load().shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim))
+def attention_prefill_shared_tiles(heads, kv_heads, head_dim, small=False) -> int:
+    """16-query tiles per workgroup of attention_prefill_shared (`small`: of its
+    variant with half as many wavefronts); 0 if the shape is not served."""
+    return int(load().shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim, int(small)))
 
 
 def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, ctx_lens, wg_seq, wg_q0,
-                             tables, k_pool, v_pool, page_size, window, scale) -> None:
+                             tables, k_pool, v_pool, page_size, window, scale, small=False) -> None:
     """bfloat16 MFMA attention for prompt portions; one workgroup per (run of query
-    tiles, key/value head) shares each chunk of keys among its query heads."""
+    tiles, key/value head) shares each chunk of keys among its query heads.
+    wg_seq / wg_q0 are in steps of 16 * attention_prefill_shared_tiles(..., small)."""
     _rows(q, "attention_prefill_shared q")
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise KernelError("attention_prefill_shared: bfloat16 only")
@@ -358,7 +360,7 @@ def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, c
             _dev(cu_q, "cu_q", torch.int32), _dev(ctx_lens, "ctx_lens", torch.int32),
             _dev(wg_seq, "wg_seq", torch.int32), _dev(wg_q0, "wg_q0", torch.int32),
             _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
-            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), _stream(),
+            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), int(small), _stream(),
         )
     )
 

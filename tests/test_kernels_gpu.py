@@ -643,13 +643,17 @@ def test_rope_kv_store_adds_up_a_split_product(ops):
     [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 128, 16, None),
      (16, 2, 64, 16, 100), (3, 1, 128, 48, None), (16, 1, 32, 16, None), (12, 1, 64, 32, 50)],
 )
-def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window):
+@pytest.mark.parametrize("small", [False, True])
+def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window, small):
     """The prefill kernel that shares each chunk of keys among the query heads of a
-    key/value head: 1 to 16 heads per group, portions of 2 to 200 tokens."""
+    key/value head: 1 to 16 heads per group, portions of 2 to 200 tokens, in
+    workgroups of 16 wavefronts and of 8 (`small`)."""
     torch.manual_seed(20)
     dtype = torch.bfloat16
-    tiles = ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim)
-    assert tiles == 16 // (heads // kv_heads)
+    tiles = ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim, small)
+    assert tiles == (8 if small else 16) // (heads // kv_heads)
+    if tiles == 0:
+        pytest.skip("more query heads per key/value head than the small workgroup has wavefronts")
     seq_lens = [2, 200, 16, 17, 90, 33, 130]
     starts = [0, 60, 5, 100, 0, 31, 7]
     ctx = [s + l for s, l in zip(starts, seq_lens)]
@@ -670,7 +674,8 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
     out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
     scale = head_dim**-0.5
     ops.attention_prefill_shared(dev(q).view(n, -1), out, len(wg_seq), heads, kv_heads, head_dim, i32(cu), i32(ctx),
-                                 i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, window, scale)
+                                 i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, window, scale,
+                                 small=small)
     want = reference_attention(q.double(), k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale)
     assert not torch.isnan(out.float()).any()
     close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
