@@ -951,23 +951,57 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
   }
 }
 
+// Estimated time in microseconds of a product of many tokens with workgroup tiles
+// of `shape` (0: 256 weight rows x 256 tokens, 1: 256 x 128, 2: 128 x 128) and
+// `split` shares of k: rounds of workgroups over the chip's 256 compute units
+// times the time of one workgroup, at the rates measured for each shape
+// (TFLOP/s per compute unit: 4.2, 3.4, and for the smallest tile 2.6 with the
+// compute unit to itself or 1.5 for each of two), plus what a kernel costs
+// anyway, plus writing and reading the float32 parts of a split product at
+// 4 TB/s.  It reproduces the measured times of the 7B and 14B matrices at 512
+// tokens within 10 %.
+static double big_estimate(int shape, int split, int n, int wblocks, int m, int k) {
+  const int rows = shape == 2 ? 128 : 256, tokens = shape == 0 ? 256 : 128;
+  const long long tiles =
+      static_cast<long long>((wblocks * 16 + rows - 1) / rows) * ((n + tokens - 1) / tokens);
+  const long long workgroups = tiles * split;
+  double rounds, rate;
+  if (shape == 2) {
+    rounds = workgroups <= 256 ? 1.0 : static_cast<double>((workgroups + 511) / 512);
+    rate = workgroups <= 256 ? 2.6 : 1.5;
+  } else {
+    rounds = static_cast<double>((workgroups + 255) / 256);
+    rate = shape == 0 ? 4.2 : 3.4;
+  }
+  const double share = static_cast<double>(k) / split;
+  double us = rounds * 2.0 * rows * tokens * share / (rate * 1e6) + 5.0;
+  if (split > 1) us += 2.0 * split * static_cast<double>(n) * m * 4.0 / 4e6;
+  return us;
+}
+
+// The shape that big_estimate() prefers for a given number of shares.
+static int big_shape(int split, int n, int wblocks, int m, int k) {
+  int best = 0;
+  for (int shape = 1; shape < 3; ++shape)
+    if (big_estimate(shape, split, n, wblocks, m, k) < big_estimate(best, split, n, wblocks, m, k))
+      best = shape;
+  return best;
+}
+
 extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   const int mblocks = (m + 15) / 16, ktiles = (k + 31) / 32;
   if (n > 64) {
-    // many tokens: tiles of 128 x 128, of which a compute unit takes one at full
-    // speed or two at 0.6 of it each.  Up to 127 tiles: as many shares of k as
-    // give every compute unit one workgroup.  128 to 191 tiles would leave a
-    // quarter of the chip idle, and two shares would give some compute units two
-    // workgroups and the others one: three shares give nearly all of them two
-    // (measured 15 to 29 % faster than one share).  Each share keeps at least 8
-    // stages of 64.
-    const long long tiles = static_cast<long long>((mblocks + 7) / 8) * ((n + 127) / 128);
-    if (tiles >= 192) return 1;
-    int split = tiles >= 128 ? 3 : static_cast<int>(256 / tiles);
-    const int most = ktiles / 16;
-    if (split > most) split = most;
-    if (split > 16) split = 16;
-    return split > 1 ? split : 1;
+    // many tokens: the number of shares, each of at least 8 stages of 64, that
+    // big_estimate() expects to be fastest with the tile shape that suits it
+    int most = ktiles / 16;
+    if (most > 16) most = 16;
+    int best = 1;
+    double least = big_estimate(big_shape(1, n, mblocks, m, k), 1, n, mblocks, m, k);
+    for (int split = 2; split <= most; ++split) {
+      const double us = big_estimate(big_shape(split, n, mblocks, m, k), split, n, mblocks, m, k);
+      if (us < 0.97 * least) least = us, best = split;  // more shares only for a clear gain
+    }
+    return best;
   }
   if (mblocks >= 512) return 1;
   // up to 16 tokens: workgroups of 4 wavefronts share a block's k-tiles; more tokens:
@@ -1004,23 +1038,12 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     SHK_REQUIRE(reinterpret_cast<uintptr_t>(out) % 8 == 0, "gemm_bf16: out is not 8-byte aligned");
     const int wblocks = (gated ? 2 : 1) * mb;  // blocks of 16 weight rows
     // Tile of the workgroup: 256 x 256, 256 x 128 or 128 x 128 (weight rows x
-    // tokens), whichever finishes first by this estimate: rounds of workgroups
-    // over the chip (256 compute units; two of the smallest tile fit on one) times
-    // the tile's work over the rate a workgroup of that shape was measured at.
-    auto rounds = [&](int rows, int tokens, int slots) {
-      const long long tiles =
-          static_cast<long long>((wblocks * 16 + rows - 1) / rows) * ((n + tokens - 1) / tokens);
-      return static_cast<double>((tiles + slots - 1) / slots);
-    };
-    const double cost_a = rounds(256, 256, 256) * (256.0 * 256.0) / 4.2;
-    const double cost_b = rounds(256, 128, 256) * (256.0 * 128.0) / 3.4;
-    // the smallest tile runs faster while it has its compute unit to itself
-    const bool c_alone = rounds(128, 128, 256) <= 1.0;
-    const double cost_c = rounds(128, 128, 512) * (128.0 * 128.0) / (c_alone ? 2.6 : 1.5);
-    if (ksplit == 1 && cost_a <= cost_b && cost_a <= cost_c)
+    // tokens), whichever big_estimate() expects to finish first.
+    const int shape = big_shape(ksplit, n, wblocks, m, k);
+    if (shape == 0)
       launch_big<4, 2, 4, 8, 1>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
-    else if (ksplit == 1 && cost_b <= cost_c)
+    else if (shape == 1)
       launch_big<4, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
     else
