@@ -429,6 +429,17 @@ __device__ __forceinline__ void big_store(const f32x4 (&acc)[WM][WN], int lane, 
                                           const float* __restrict__ bias, void* __restrict__ out,
                                           int ldo, int out_f32, int accumulate, int share) {
   const int j = lane % 16, kg = lane / 16;
+  // the lane's bias values, fetched once for all its tokens
+  float add[GATED ? 1 : WM][4];
+  if (!GATED) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = (block_first + i) * 16 + kg * 4 + r;
+        add[i][r] = (bias && row < m) ? bias[row] : 0.f;
+      }
+  }
 #pragma unroll
   for (int jn = 0; jn < WN; ++jn) {
     const int token = tok_first + jn * 16 + j;
@@ -441,8 +452,8 @@ __device__ __forceinline__ void big_store(const f32x4 (&acc)[WM][WN], int lane, 
       float v[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r] : acc[i][jn][r];
-        if (bias && row0 + r < m) v[r] += bias[row0 + r];
+        v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r]
+                     : acc[i][jn][r] + add[GATED ? 0 : i][r];
       }
       const size_t idx = (static_cast<size_t>(share) * n + token) * ldo + row0;
       if (out_f32) {
