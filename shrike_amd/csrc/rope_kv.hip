@@ -133,6 +133,145 @@ __global__ void __launch_bounds__(kRopeThreads)
   }
 }
 
+// The same for bfloat16 rows that are rotated whole (rot_dim == head_dim, a
+// multiple of 16): one workgroup per token, a thread moves 8 neighbouring
+// elements at a time (16 bytes; a rotated pair is two such runs, head_dim / 2
+// apart), so that queries and keys travel in whole vectors.  Values go to
+// their transposed pages element by element.  Arithmetic as above.
+constexpr int kVecItems = 4;  // runs (or pairs of runs) per thread at most
+// from this many tokens on; fewer (decode steps) are a matter of latency, which the
+// kernel above with its ten workgroups per token and eight parts in flight handles better
+constexpr int kVecMinTokens = 65;
+
+__global__ void __launch_bounds__(kRopeThreads)
+    rope_kv_store_vec_kernel(bf16* __restrict__ qkv, int n, int heads, int kv_heads, int head_dim,
+                             const float* __restrict__ inv_freq,
+                             const int32_t* __restrict__ positions,
+                             const int32_t* __restrict__ token_seq,
+                             const int32_t* __restrict__ tables, int table_stride,
+                             bf16* __restrict__ k_pool, bf16* __restrict__ v_pool, int page_size,
+                             int num_pages, int write_kv, const float* __restrict__ parts, int splits,
+                             const float* __restrict__ bias) {
+  __shared__ float cs[kMaxHalf];
+  __shared__ float sn[kMaxHalf];
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = head_dim / 2;
+  const int width = (heads + 2 * kv_heads) * head_dim;
+  bf16* row = qkv + static_cast<size_t>(t) * width;
+  const int per_head = half / 8;                      // pairs of runs in a rotated head
+  const int n_pairs = (heads + kv_heads) * per_head;  // queries, then keys
+  const int n_values = kv_heads * (head_dim / 8);
+  const size_t split_stride = static_cast<size_t>(n) * width;
+
+  // 8 elements from column `col` on: the row itself, or the sum of its parts and the bias
+  auto fetch = [&](int col, float (&x)[8]) {
+    if (splits == 0) {
+      const uint4 raw = *reinterpret_cast<const uint4*>(row + col);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[2 * e] = __uint_as_float(w[e] << 16);
+        x[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
+      }
+      return;
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = 0.f;
+    const float* p = parts + static_cast<size_t>(t) * width + col;
+    for (int z0 = 0; z0 < splits; z0 += 4) {  // four parts in flight, added in order
+      float4 lo[4], hi[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int z = z0 + u < splits ? z0 + u : splits - 1;
+        lo[u] = *reinterpret_cast<const float4*>(p + z * split_stride);
+        hi[u] = *reinterpret_cast<const float4*>(p + z * split_stride + 4);
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const bool have = z0 + u < splits;  // (past the last part: the last one again, not added)
+        x[0] += have ? lo[u].x : 0.f, x[1] += have ? lo[u].y : 0.f;
+        x[2] += have ? lo[u].z : 0.f, x[3] += have ? lo[u].w : 0.f;
+        x[4] += have ? hi[u].x : 0.f, x[5] += have ? hi[u].y : 0.f;
+        x[6] += have ? hi[u].z : 0.f, x[7] += have ? hi[u].w : 0.f;
+      }
+    }
+    if (bias) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) x[e] += bias[col + e];
+    }
+  };
+  auto pack = [](const float (&x)[8]) {
+    uint4 out;
+    out.x = bf16_bits(x[0]) | (static_cast<uint32_t>(bf16_bits(x[1])) << 16);
+    out.y = bf16_bits(x[2]) | (static_cast<uint32_t>(bf16_bits(x[3])) << 16);
+    out.z = bf16_bits(x[4]) | (static_cast<uint32_t>(bf16_bits(x[5])) << 16);
+    out.w = bf16_bits(x[6]) | (static_cast<uint32_t>(bf16_bits(x[7])) << 16);
+    return out;
+  };
+
+  // this thread's items, fetched before the table of cosines and sines is made
+  float a[kVecItems][8], b[kVecItems][8];
+#pragma unroll
+  for (int u = 0; u < kVecItems; ++u) {
+    const int item = threadIdx.x + u * kRopeThreads;
+    if (item < n_pairs) {
+      const int col = (item / per_head) * head_dim + (item % per_head) * 8;
+      fetch(col, a[u]);
+      fetch(col + half, b[u]);
+    } else if (item < n_pairs + n_values) {
+      fetch((heads + kv_heads) * head_dim + (item - n_pairs) * 8, a[u]);
+    }
+  }
+
+  int page = -1;
+  if (write_kv) {
+    page = tables[static_cast<size_t>(token_seq[t]) * table_stride + pos / page_size];
+    if (page < 0 || page >= num_pages) page = -1;  // a host bug; never dereferenced
+  }
+  const int slot = pos % page_size;
+  const size_t page_base = static_cast<size_t>(page < 0 ? 0 : page) * kv_heads * page_size * head_dim;
+
+  for (int f = threadIdx.x; f < half; f += kRopeThreads) {
+    const float angle = static_cast<float>(pos) * inv_freq[f];
+    const double wide = static_cast<double>(angle);
+    const double turns = rint(wide * 0.15915494309189535);
+    const float reduced = static_cast<float>(fma(turns, -6.283185307179586, wide));
+    float sv, cv;
+    sincosf(reduced, &sv, &cv);
+    cs[f] = cv;
+    sn[f] = sv;
+  }
+  __syncthreads();
+
+#pragma unroll
+  for (int u = 0; u < kVecItems; ++u) {
+    const int item = threadIdx.x + u * kRopeThreads;
+    if (item < n_pairs) {
+      const int h = item / per_head, i = (item % per_head) * 8;
+      float lo[8], hi[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        lo[e] = a[u][e] * cs[i + e] - b[u][e] * sn[i + e];
+        hi[e] = b[u][e] * cs[i + e] + a[u][e] * sn[i + e];
+      }
+      if (h < heads) {
+        *reinterpret_cast<uint4*>(row + h * head_dim + i) = pack(lo);
+        *reinterpret_cast<uint4*>(row + h * head_dim + i + half) = pack(hi);
+      } else if (page >= 0) {
+        bf16* dst = k_pool + page_base + static_cast<size_t>(h - heads) * page_size * head_dim;
+        *reinterpret_cast<uint4*>(dst + key_offset(slot, i, page_size, head_dim)) = pack(lo);
+        *reinterpret_cast<uint4*>(dst + key_offset(slot, i + half, page_size, head_dim)) = pack(hi);
+      }
+    } else if (item < n_pairs + n_values && page >= 0) {
+      const int d0 = (item - n_pairs) * 8;  // kv head * head_dim + element
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        v_pool[page_base + static_cast<size_t>(d0 + e) * page_size + slot] = from_float<bf16>(a[u][e]);
+    }
+  }
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -164,10 +303,23 @@ extern "C" int shk_rope_kv_store(void* qkv, int dtype, int n, int heads, int kv_
                 "rope_kv_store: bad cache sizes page_size=%d num_pages=%d table_stride=%d",
                 page_size, num_pages, table_stride);
   }
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // whole vectors where the layout allows: bfloat16, rows rotated whole, 16-byte alignment
+  const int vec_items = (heads + kv_heads) * (head_dim / 16) + kv_heads * (head_dim / 8);
+  if (dtype == kBF16 && rot_dim == head_dim && head_dim % 16 == 0 && n >= kVecMinTokens &&
+      vec_items <= kVecItems * kRopeThreads && reinterpret_cast<uintptr_t>(qkv) % 16 == 0 &&
+      (!write_kv || reinterpret_cast<uintptr_t>(k_pool) % 16 == 0) &&
+      (!parts || reinterpret_cast<uintptr_t>(parts) % 16 == 0)) {
+    rope_kv_store_vec_kernel<<<n, kRopeThreads, 0, s>>>(
+        static_cast<bf16*>(qkv), n, heads, kv_heads, head_dim, inv_freq, positions, token_seq, tables,
+        table_stride, static_cast<bf16*>(k_pool), static_cast<bf16*>(v_pool), page_size, num_pages,
+        write_kv, parts, splits, bias);
+    SHK_LAUNCH_CHECK("rope_kv_store");
+    return 0;
+  }
   const int items = (heads + kv_heads) * (head_dim - rot_dim / 2) + kv_heads * head_dim;
   dim3 grid(n, (items + kRopeThreads - 1) / kRopeThreads);
   SHK_REQUIRE(grid.y <= 65535, "rope_kv_store: too many elements per token");
-  hipStream_t s = static_cast<hipStream_t>(stream);
   if (dtype == kF32)
     rope_kv_store_kernel<float><<<grid, kRopeThreads, 0, s>>>(
         static_cast<float*>(qkv), n, heads, kv_heads, head_dim, rot_dim, inv_freq, positions,

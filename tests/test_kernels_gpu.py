@@ -142,10 +142,11 @@ def paged_setup(seq_lens, page_size, num_pages, kv_heads, head_dim, dtype, seed=
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads, kv_heads, head_dim, page_size, theta", [(6, 3, 48, 8, 5e4), (14, 2, 64, 16, 1e6), (5, 5, 80, 4, 1e4)])
+@pytest.mark.parametrize("heads, kv_heads, head_dim, page_size, theta", [(6, 3, 48, 8, 5e4), (14, 2, 64, 16, 1e6), (5, 5, 80, 4, 1e4),
+                                                                   (4, 2, 128, 16, 1e6), (3, 1, 72, 8, 1e4)])
 def test_rope_kv_store(ops, dtype, heads, kv_heads, head_dim, page_size, theta):
     torch.manual_seed(6)
-    seq_lens = [37, 1, 12]
+    seq_lens = [37, 1, 40]  # 78 tokens: bfloat16 rows that are rotated whole take the vector kernel
     starts = [5, 0, 3000]  # positions far out: angles of thousands of radians
     n = sum(seq_lens)
     tables, k_pool, v_pool = paged_setup([s + l for s, l in zip(starts, seq_lens)], page_size, 1024, kv_heads, head_dim, dtype)
@@ -607,17 +608,17 @@ def test_split_product_and_its_readers(ops, n, m, k):
         close(out, plain.rms_norm((before + total).double().cpu(), wn.double().cpu(), 1e-5), dtype)
 
 
-def test_rope_kv_store_adds_up_a_split_product(ops):
+@pytest.mark.parametrize("n, splits", [(5, 3), (70, 3), (66, 9)])  # few tokens: element by element; many: in vectors
+def test_rope_kv_store_adds_up_a_split_product(ops, n, splits):
     torch.manual_seed(19)
     dtype = torch.bfloat16
     heads, kv_heads, head_dim, page_size, theta = 6, 2, 64, 16, 1e4
-    n, splits = 5, 3
     width = (heads + 2 * kv_heads) * head_dim
     parts = torch.randn(splits, n, width, device="cuda")
     bias = torch.randn(width, device="cuda")
-    positions = torch.tensor([3, 17, 100, 0, 31], dtype=torch.int32, device="cuda")
+    positions = torch.tensor([3, 17, 100, 0, 31] + list(range(40, 35 + n)), dtype=torch.int32, device="cuda")
     token_seq = torch.arange(n, dtype=torch.int32, device="cuda")
-    tables, k_pool, v_pool = paged_setup([p + 1 for p in positions.tolist()], page_size, 32, kv_heads, head_dim, dtype)
+    tables, k_pool, v_pool = paged_setup([p + 1 for p in positions.tolist()], page_size, 512, kv_heads, head_dim, dtype)
     inv_freq = (1.0 / (theta ** (torch.arange(0, head_dim, 2).float() / head_dim))).cuda()
     qkv = torch.full((n, width), float("nan"), device="cuda", dtype=dtype)
     ops.rope_kv_store(qkv, heads, kv_heads, head_dim, head_dim, inv_freq, positions, token_seq, tables,
