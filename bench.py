@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L] [--shape 7b]
+    python bench.py --shape 14b --mixed 32      # a mixed step instead (a line of its own)
 
 The model has the layer sizes of the Qwen2.5-7B shape (28 layers, hidden 3584,
 28 query heads over 4 key/value heads of 128, intermediate 18944, vocabulary
@@ -82,7 +83,7 @@ def prefill_flops(cfg, n: int) -> float:
     return linear + attn
 
 
-def make_engine(cfg, spec, max_batch: int, seed: int):
+def make_engine(cfg, spec, max_batch: int, seed: int, budget: int | None = None):
     import torch
 
     from shrike_amd.config import EngineConfig
@@ -95,7 +96,8 @@ def make_engine(cfg, spec, max_batch: int, seed: int):
     print(f"[bench] random weights on the device in {time.perf_counter() - t0:.1f}s", file=sys.stderr)
     pages = max_batch * (CONTEXT_END // PAGE_SIZE + 2)
     config = EngineConfig(
-        block_size=PAGE_SIZE, num_kv_blocks=pages, max_tokens_per_step=PROMPT_LEN + max_batch,
+        block_size=PAGE_SIZE, num_kv_blocks=pages,
+        max_tokens_per_step=budget if budget is not None else PROMPT_LEN + max_batch,
         max_running=max_batch, enable_prefix_caching=False, dtype="bfloat16", seed=seed,
     )
     return LLMEngine(None, config, model=model, runtime=runtime)
@@ -160,6 +162,47 @@ def run_prefill(engine, cfg, seed: int, repeats: int = 3) -> dict:
             "frac": round(flops / best / BF16_PEAK_FLOPS, 4)}
 
 
+def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
+    """`decodes` requests decoding at a context of about PROMPT_LEN while one more
+    PROMPT_LEN-token prompt is admitted under a token budget of `budget` a step:
+    the time of the steps that hold `decodes` single tokens and a prompt portion."""
+    import torch
+
+    from shrike_amd import SamplingParams
+
+    rng = random.Random(seed)
+    sampling = SamplingParams(max_new_tokens=400, ignore_eos=True)
+    for _ in range(decodes):
+        engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)], sampling)
+    while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
+        engine.step()
+    for _ in range(20):
+        engine.step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(50):
+        engine.step()
+    torch.cuda.synchronize()
+    decode_ms = (time.perf_counter() - t0) / 50 * 1e3
+    engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)],
+                       SamplingParams(max_new_tokens=8, ignore_eos=True))
+    full = []  # steps that use the whole budget
+    while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
+        left = max(r.num_tokens - r.num_computed_tokens for r in list(engine.scheduler.waiting) +
+                   engine.scheduler.running)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step()
+        torch.cuda.synchronize()
+        if left >= budget - decodes:
+            full.append((time.perf_counter() - t0) * 1e3)
+    for req in list(engine.scheduler.running):
+        engine.abort(req.req_id)
+    mean = sum(full) / len(full)
+    return {"decode_only_ms": round(decode_ms, 3), "mixed_step_ms": round(mean, 3), "mixed_steps": len(full),
+            "tokens_per_s": round(budget / mean * 1e3, 1)}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
@@ -172,6 +215,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b",
                     help="layer sizes: Qwen2.5-7B (the default and the reported figure), 14B or 32B")
+    ap.add_argument("--mixed", type=int, default=0, metavar="DECODES",
+                    help="instead: time steps of DECODES single tokens plus a portion of a 2,048-token "
+                         "prompt under a 512-token budget (prints its own JSON line)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -196,6 +242,20 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
+    if args.mixed:
+        engine = make_engine(cfg, spec, args.mixed + 1, args.seed, budget=512)
+        mixed = run_mixed(engine, cfg, args.mixed, 512, args.seed)
+        print(json.dumps({
+            "metric": f"ms of a step of {args.mixed} decodes plus a prompt portion, 512-token budget "
+                      f"(Qwen2.5-{args.shape.upper()} shape)",
+            "value": mixed["mixed_step_ms"], "unit": "ms", "n_gpus": 1, "higher_is_better": False,
+            "dtype": "bf16", "data": "synthetic: random weights N(0, 0.02), prompt ids uniform in [0, vocab)",
+            "config": {"model": f"Qwen2.5-{args.shape.upper()} shape (Qwen2ForCausalLM)",
+                       "layers": cfg.num_hidden_layers, "layers_of_config": layers_of_config,
+                       "decodes": args.mixed, "token_budget": 512, "prompt_len": PROMPT_LEN,
+                       "page_size": PAGE_SIZE},
+            **mixed}))
+        return 0
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     engine = make_engine(cfg, spec, max(batches), args.seed)
 
