@@ -717,7 +717,7 @@ __global__ void __launch_bounds__(GM* GN* kWave)
 #define SHK_WAIT_LOADS(n) __builtin_amdgcn_s_waitcnt(0x0f70 | ((n) & 15) | (((n) >> 4) << 14))
 
 template <int GM, int GN, int WM, int WN, int KS, bool GATED>
-__global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per_eu(2)))
+__global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per_eu(GM * GN >= 16 ? 4 : 2)))
     gemm_big_lds_kernel(const bf16* __restrict__ a, int lda, int n, int k,
                         const uint4* __restrict__ wt, int ktiles, int m,
                         const float* __restrict__ bias, void* __restrict__ out, int ldo,
@@ -966,7 +966,7 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
 // of `shape` (0: 256 weight rows x 256 tokens, 1: 256 x 128, 2: 128 x 128) and
 // `split` shares of k: rounds of workgroups over the chip's 256 compute units
 // times the time of one workgroup, at the rates measured for each shape
-// (TFLOP/s per compute unit: 4.2, 3.4, and for the smallest tile 2.6 with the
+// (TFLOP/s per compute unit: 4.2, 3.4, and for the smallest tile 3.0 with the
 // compute unit to itself or 1.5 for each of two), plus what a kernel costs
 // anyway, plus writing and reading the float32 parts of a split product at
 // 4 TB/s.  It reproduces the measured times of the 7B and 14B matrices at 512
@@ -979,7 +979,7 @@ static double big_estimate(int shape, int split, int n, int wblocks, int m, int 
   double rounds, rate;
   if (shape == 2) {
     rounds = workgroups <= 256 ? 1.0 : static_cast<double>((workgroups + 511) / 512);
-    rate = workgroups <= 256 ? 2.6 : 1.5;
+    rate = workgroups <= 256 ? 3.0 : 1.5;
   } else {
     rounds = static_cast<double>((workgroups + 255) / 256);
     rate = shape == 0 ? 4.2 : 3.4;
@@ -1052,12 +1052,16 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     // tokens), whichever big_estimate() expects to finish first.
     const int shape = big_shape(ksplit, n, wblocks, m, k);
     if (shape == 0)
-      launch_big<4, 2, 4, 8, 1>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+      launch_big<4, 4, 4, 4, 1>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
     else if (shape == 1)
-      launch_big<4, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+      launch_big<4, 4, 4, 2, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
-    else
+    else if (static_cast<long long>((wblocks + 7) / 8) * ((n + 127) / 128) * ksplit <= 256)
+      // every workgroup has a compute unit to itself: eight wavefronts, loads straight into LDS
+      launch_big<4, 2, 2, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
+                                gated, wblocks, ksplit);
+    else  // four wavefronts and two LDS buffers: two workgroups fit on a compute unit
       launch_big<2, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
     SHK_LAUNCH_CHECK("gemm_bf16");

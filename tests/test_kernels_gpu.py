@@ -580,7 +580,7 @@ def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
 
 @pytest.mark.parametrize("n, m, k", [(8, 3584, 3584), (1, 48, 4000), (33, 200, 1600), (64, 100, 2100),
                                      (100, 3584, 3584), (300, 136, 1100), (64, 2100, 16400), (40, 2100, 16400),
-                                     (256, 8192, 1600)])  # the last: 128 tiles, three shares
+                                     (512, 5120, 5120)])  # the last: many tokens, tiles of 256 x 128 in three shares
 def test_split_product_and_its_readers(ops, n, m, k):
     """A product split along k leaves partial sums; the norm and the cache-write
     kernel add them up in order and give what the unsplit product gives."""
