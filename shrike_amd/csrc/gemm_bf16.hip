@@ -966,7 +966,7 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
 // of `shape` (0: 256 weight rows x 256 tokens, 1: 256 x 128, 2: 128 x 128) and
 // `split` shares of k: rounds of workgroups over the chip's 256 compute units
 // times the time of one workgroup, at the rates measured for each shape
-// (TFLOP/s per compute unit: 4.2, 3.4, and for the smallest tile 3.0 with the
+// (TFLOP/s per compute unit: 4.75, 4.0, and for the smallest tile 3.0 with the
 // compute unit to itself or 1.5 for each of two), plus what a kernel costs
 // anyway, plus writing and reading the float32 parts of a split product at
 // 4 TB/s.  It reproduces the measured times of the 7B and 14B matrices at 512
@@ -982,7 +982,7 @@ static double big_estimate(int shape, int split, int n, int wblocks, int m, int 
     rate = workgroups <= 256 ? 3.0 : 1.5;
   } else {
     rounds = static_cast<double>((workgroups + 255) / 256);
-    rate = shape == 0 ? 4.2 : 3.4;
+    rate = shape == 0 ? 4.75 : 4.0;
   }
   const double share = static_cast<double>(k) / split;
   double us = rounds * 2.0 * rows * tokens * share / (rate * 1e6) + 5.0;
