@@ -801,8 +801,10 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
       u32x4 x = held[i];
-      if (!is_k[i]) {
-        // keys outside [lo_min, pos_max] carry weight 0, but their slots may hold anything
+      // keys outside [lo_min, pos_max] carry weight 0, but their slots may hold anything;
+      // only the first and the last chunk have such keys
+      if (!is_k[i] && (kb < lo_min || kb + 31 > pos_max)) {
+        asm volatile("");  // stays a branch: as selects the comparisons would run for every chunk
         u32x4 keep;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -846,6 +848,9 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
 #pragma unroll
       for (int e = 0; e < 8; ++e) sc[e] = s[e / 4][e % 4] * scale2;
       if (edge) {  // wave-uniform: some query of the workgroup does not read the whole chunk
+        // (the empty statement keeps this a branch: turned into selects, the
+        // comparisons would run for every chunk)
+        asm volatile("");
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           if (g0 + e > q_pos[u] || g0 + e < q_lo[u]) sc[e] = -INFINITY;
