@@ -260,6 +260,15 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
   }
 }
 
+// max(a, b, c) in one instruction.  Written out because fmaxf() first quiets each
+// operand that might be a signalling NaN (one more instruction per operand), which
+// scores, being products or -inf, never are.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // ------------------------------------------------------------------- decode
 // grid (kv_heads, sequences, splits), kDecodeWaves wavefronts per workgroup.  A
 // single wavefront needs about 1,700 cycles for a chunk of 32 keys whatever the
@@ -407,8 +416,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
         for (int e = 0; e < 8; ++e)
           if (g0 + e > pos || g0 + e < lo) sc[e] = -INFINITY;
       }
-      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                       fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      float mx = max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), fmaxf(sc[6], sc[7]));
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
       const float m_new = fmaxf(m, mx);
@@ -855,8 +863,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
         for (int e = 0; e < 8; ++e)
           if (g0 + e > q_pos[u] || g0 + e < q_lo[u]) sc[e] = -INFINITY;
       }
-      float mx = fmaxf(fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3])),
-                       fmaxf(fmaxf(sc[4], sc[5]), fmaxf(sc[6], sc[7])));
+      float mx = max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), fmaxf(sc[6], sc[7]));
       mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
       mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
       const float m_new = fmaxf(m[u], mx);
