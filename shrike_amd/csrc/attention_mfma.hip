@@ -262,7 +262,11 @@ __device__ __forceinline__ void attend_tile(const TileArgs& ta, const AFrag (&qf
 
 // max(a, b, c) in one instruction.  Written out because fmaxf() first quiets each
 // operand that might be a signalling NaN (one more instruction per operand), which
-// scores, being products or -inf, never are.
+// scores, being products or -inf, never are.  The operands must come from vector
+// instructions, never straight from a matrix instruction: the compiler does not
+// count the wait states that a matrix result needs for an instruction it cannot
+// see into (scores scaled inside the exponent, and so fed unscaled from the
+// matrix unit into this, came out wrong).
 __device__ __forceinline__ float max3(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
