@@ -986,7 +986,9 @@ static double big_estimate(int shape, int split, int n, int wblocks, int m, int 
   }
   const double share = static_cast<double>(k) / split;
   double us = rounds * 2.0 * rows * tokens * share / (rate * 1e6) + 5.0;
-  if (split > 1) us += 2.0 * split * static_cast<double>(n) * m * 4.0 / 4e6;
+  // (tokens counted in whole tiles of 128: the choice is then the same for every
+  // number of tokens that a captured decode step of 128 or 256 rows may stand for)
+  if (split > 1) us += 2.0 * split * ((n + 127) / 128 * 128.0) * m * 4.0 / 4e6;
   return us;
 }
 

@@ -88,3 +88,45 @@ def test_one_layer_of_the_7b_shape(dtype, tol, model_dir, reference):
         for other in (tail, portions, mixed):
             assert rel_err(other, whole) <= 1e-5
     cache.check([])
+
+
+@pytest.mark.parametrize("count", [100, 150])
+def test_many_single_tokens_as_a_graph_and_kernel_by_kernel(model_dir, count):
+    """100 or 150 sequences decode together (graphs of 128 and 256 rows): a batch that the large product kernels
+    serve (tiles of 128 and 256 tokens, operands loaded straight into LDS, shares
+    of k).  Replayed from a HIP graph several times, with the program's own work
+    between the replays, the logits equal those of kernel-by-kernel execution
+    bit for bit."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    model, rt, _ = load_model(model_dir, "bfloat16")
+    rng = random.Random(11)
+    prompts = [[rng.randrange(SHAPE["vocab_size"]) for _ in range(rng.randint(1, 5))] for _ in range(count)]
+    feed = [[rng.randrange(SHAPE["vocab_size"]) for _ in range(4)] for _ in range(count)]
+
+    def run(graphs):
+        cache = CacheManager(model.cache_specs(), 16, 160, enable_prefix_caching=False)
+        cache.allocate(rt.dtype, rt.device)
+        runner = ModelRunner(model, cache, rt, graphs=graphs)
+        seqs = [cache.new_sequence() for _ in prompts]
+        for s, p in zip(seqs, prompts):
+            cache.append(s, 0, len(p))
+        runner.step([StepEntry(s, p, 0, []) for s, p in zip(seqs, prompts)])
+        outs = []
+        for step in range(4):
+            entries = []
+            for s, p, f in zip(seqs, prompts, feed):
+                cache.append(s, len(p) + step, 1)
+                entries.append(StepEntry(s, [f[step]], len(p) + step, [0]))
+            outs.append(runner.step(entries).clone())
+            torch.cuda.synchronize()
+        assert runner.graph_replays == (4 if graphs else 0)
+        for s in seqs:
+            cache.free(s)
+        return outs
+
+    eager, replayed = run(False), run(True)
+    for a, b in zip(eager, replayed):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
