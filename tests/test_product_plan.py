@@ -32,3 +32,19 @@ def test_matrices_that_fill_the_chip_are_not_split():
     assert ops.gemm_splits(4096, 18944, 3584) == 1    # 592 tiles of 256 x 256
     assert ops.gemm_splits(8, 3584, 18944) > 1        # 224 row blocks, a long k
     assert ops.gemm_splits(512, 5120, 13824) > 1      # 80 tiles of 256 x 128
+
+
+def test_key_splits_of_decode_attention_depend_on_the_buckets_only():
+    """A graph is captured for a bucket of sequences and of context; every step
+    that it replays must split the keys as the captured one did."""
+    from shrike_amd.engine.runtime import bucket, decode_splits
+
+    for kv_heads in (1, 4, 8):
+        for seqs_lo, seqs_hi in ((1, 1), (3, 4), (5, 8), (33, 64), (129, 256)):
+            for ctx_lo, ctx_hi in ((1, 256), (257, 512), (2049, 4096), (16385, 32768)):
+                plans = {decode_splits(s, kv_heads, c)
+                         for s in (seqs_lo, seqs_hi) for c in (ctx_lo, (ctx_lo + ctx_hi) // 2, ctx_hi)}
+                assert len(plans) == 1
+                (n,) = plans
+                assert 1 <= n <= 64 and n <= max(1, bucket(ctx_hi, 256) // 256)
+    assert decode_splits(8, 4, 2100) == 8 and decode_splits(64, 4, 4000) == 1 and decode_splits(1, 4, 100) == 1
