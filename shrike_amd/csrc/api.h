@@ -68,9 +68,11 @@ int shk_gemm_bf16_splits(int n, int m, int k);
 // keys are rotated by position (pairs (i, i + rot_dim/2), angle position *
 // inv_freq[i]); queries are rewritten in place; keys and values go to their
 // page slots: page = tables[token_seq[t] * table_stride + position / page_size].
-// The key pool is [num_pages, kv_heads, page_size, head_dim]; the value pool is
-// stored transposed, [num_pages, kv_heads, head_dim, page_size].  rot_dim 0
-// rotates nothing; write_kv 0 leaves the pools alone.
+// The key pool holds each page's keys in slabs of 32 elements, [num_pages,
+// kv_heads, head_dim / 32, page_size, 32] (one slab of head_dim elements where
+// head_dim is no multiple of 32); the value pool is stored transposed,
+// [num_pages, kv_heads, head_dim, page_size].  rot_dim 0 rotates nothing;
+// write_kv 0 leaves the pools alone.
 // splits > 0: the projections come as float32 partial sums `parts`
 // [splits][n][width] of a product split along k; they are added in order, `bias`
 // (float32 [width] or null) is added, and the rotated queries are written to

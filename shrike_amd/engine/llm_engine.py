@@ -69,6 +69,7 @@ class LLMEngine:
         self.sampler = Sampler(runtime.device, cfg.seed)
         self.eos_ids = set(model.spec.eos_token_ids)
         self.requests: dict[int, Request] = {}
+        self._next_req_id = 0
         self.stats = EngineStats()
         # (batch, prepared step) of the next step, laid out while the device ran the last
         # one; dropped whenever a request arrives, ends or is aborted
@@ -101,7 +102,8 @@ class LLMEngine:
                 f"only {self.cache.num_pages}; it could never be scheduled - shorten the prompt, "
                 "lower max_new_tokens, or raise gpu_mem_util / num_kv_blocks"
             )
-        req = Request(token_ids=token_ids, sampling=sampling)
+        req = Request(token_ids=token_ids, sampling=sampling, req_id=self._next_req_id)
+        self._next_req_id += 1
         self.requests[req.req_id] = req
         self.scheduler.add(req)
         self._planned = None

@@ -38,22 +38,27 @@ class SamplingParams:
     seed: int | None = None
 
     def __post_init__(self) -> None:
+        problems = []
         if self.max_new_tokens < 1:
-            raise ValueError(f"max_new_tokens must be >= 1, got {self.max_new_tokens}")
+            problems.append(f"max_new_tokens={self.max_new_tokens} (at least one token must be generated)")
         if self.temperature < 0.0:
-            raise ValueError(f"temperature must be >= 0, got {self.temperature}")
+            problems.append(f"temperature={self.temperature} (negative; 0 means greedy)")
         if not 0.0 < self.top_p <= 1.0:
-            raise ValueError(f"top_p must be in (0, 1], got {self.top_p}")
+            problems.append(f"top_p={self.top_p} (the nucleus mass lies in (0, 1])")
+        if problems:
+            raise ValueError("bad sampling parameters: " + "; ".join(problems))
 
 
-_req_counter = itertools.count()
+# ids of requests made outside an engine (an engine numbers its own from 0, so
+# that its default sampling seeds do not depend on what else the process ran)
+_loose_ids = itertools.count()
 
 
 @dataclass
 class Request:
     token_ids: list[int]  # prompt; generated tokens are appended in place
     sampling: SamplingParams
-    req_id: int = field(default_factory=lambda: next(_req_counter))
+    req_id: int = field(default_factory=_loose_ids.__next__)
     status: Status = Status.WAITING
     num_prompt_tokens: int = 0
     num_computed_tokens: int = 0  # tokens whose keys/values are in the cache

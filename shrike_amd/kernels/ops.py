@@ -234,8 +234,8 @@ def _check_pools(who, q, tables, k_pool, v_pool, kv_heads, head_dim, page_size) 
 def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, token_seq,
                   tables, k_pool, v_pool, page_size, write_kv=True, split_sum=None) -> None:
     """Rotate q and k of qkv [n, (heads + 2 kv_heads) head_dim] in float32 and put
-    k, v into their pages (keys [pages, kv_heads, page_size, head_dim], values
-    transposed [pages, kv_heads, head_dim, page_size])."""
+    k, v into their pages (keys in slabs, see key_pool_shape; values transposed
+    [pages, kv_heads, head_dim, page_size])."""
     n = qkv.shape[0]
     if not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
         raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim]")

@@ -1,7 +1,7 @@
 """Plain, slow implementation of the Qwen2.5 dense decoder on the CPU.
 
 Whole sequences, no cache, one function for each part, written from the
-formulas of the reference (cited as ``path:line`` under /root/reference).
+formulas of the reference (cited as ``path:line`` of Azimml/shrike's tree).
 It shares no code with the product path: it parses config.json and reads
 model.safetensors by itself and uses only torch tensor arithmetic.
 
