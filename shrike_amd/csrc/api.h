@@ -140,6 +140,18 @@ int shk_argmax(const float* logits, int32_t* out, int rows, int vocab, int ld, f
                void* stream);
 int shk_argmax_scratch_floats(int rows, int vocab);
 
+// shk_argmax for callers that cannot allocate device memory or bring a workspace
+// (code recorded into a HIP graph, tight serving loops, harnesses that forbid
+// hipMalloc).  It has no counterpart in the reference.  The chunk results live
+// in an array of shk_argmax_static_max_floats() floats (256 KiB) that the library
+// holds on every GPU it runs on until the process ends; a call whose
+// shk_argmax_scratch_floats(rows, vocab) exceeds that is refused.  No call
+// allocates or frees anything.  All calls on one GPU share that GPU's array:
+// calls that overlap there (two streams, two threads) race; calls in stream order
+// do not, and nothing an earlier call left in the array is read.
+int shk_argmax_static(const float* logits, int32_t* out, int rows, int vocab, int ld, void* stream);
+int shk_argmax_static_max_floats(void);
+
 // Temperature / top-p sampling of one token per row (see sampling.hip).
 // temperature[r] == 0 takes the argmax.  uniforms[r] in [0, 1) is the draw.
 // `scratch` is float32 [rows, vocab].

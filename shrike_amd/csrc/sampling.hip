@@ -10,6 +10,8 @@
 // x; entries equal to tau are kept lowest index first, as many as the rule
 // admits.  The draw walks the kept entries in index order with the caller's
 // uniform number, so a row's result depends only on its logits and its number.
+#include <mutex>
+
 #include "api.h"
 #include "common.h"
 
@@ -245,6 +247,56 @@ extern "C" int shk_argmax(const float* logits, int32_t* out, int rows, int vocab
   argmax_pick_kernel<<<rows, kArgmaxThreads, 0, s>>>(best_value, best_index, out, chunks);
   SHK_LAUNCH_CHECK("argmax");
   return 0;
+}
+
+// ------------------------------------------------------ argmax without a workspace
+// The chunk results of the two-stage argmax in memory that the library itself
+// holds: one array per GPU, there from the moment the code object is loaded until
+// the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels get the device address it returns.
+constexpr int kStaticScratchFloats = 1 << 16;  // 256 KiB: 2 * rows * chunks floats at most
+static __device__ __align__(256) float scratch[kStaticScratchFloats];
+
+constexpr int kMaxDevices = 64;
+static std::mutex scratch_mutex;
+static float* scratch_of_device[kMaxDevices];  // device address of `scratch` on each GPU
+
+// Address of the current device's copy of `scratch`, looked up once per device.
+static int static_scratch(float** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  SHK_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  SHK_REQUIRE(device >= 0 && device < kMaxDevices, "argmax_static: device %d is beyond %d", device,
+              kMaxDevices);
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (scratch_of_device[device] == nullptr) {
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    SHK_REQUIRE(e == hipSuccess && addr != nullptr,
+                "argmax_static: hipGetSymbolAddress failed on device %d: %s", device,
+                hipGetErrorString(e));
+    scratch_of_device[device] = static_cast<float*>(addr);
+  }
+  *ptr = scratch_of_device[device];
+  return 0;
+}
+
+extern "C" int shk_argmax_static_max_floats(void) { return kStaticScratchFloats; }
+
+extern "C" int shk_argmax_static(const float* logits, int32_t* out, int rows, int vocab, int ld,
+                                 void* stream) {
+  SHK_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab,
+              "argmax_static: bad sizes rows=%d vocab=%d ld=%d", rows, vocab, ld);
+  const long long need = shk_argmax_scratch_floats(1, vocab) * static_cast<long long>(rows);
+  SHK_REQUIRE(need <= kStaticScratchFloats,
+              "argmax_static: %d rows of %d values need %lld floats of scratch, the library's own "
+              "array holds %d (use shk_argmax with a workspace)",
+              rows, vocab, need, kStaticScratchFloats);
+  float* ptr = nullptr;
+  if (int rc = static_scratch(&ptr)) return rc;
+  // every chunk result that the second kernel reads is written by the first one in
+  // this call: nothing has to be cleared, whatever an earlier call left behind
+  return shk_argmax(logits, out, rows, vocab, ld, ptr, stream);
 }
 
 extern "C" int shk_sample(const float* logits, int32_t* out, const float* temperature,
