@@ -47,6 +47,10 @@ class LayerCache:
     v_pool: object = None
     window: int | None = None
     state: object = None  # [slots, *shape] for a StateSpec layer
+    # the same memory with one slot more, [slots + 1, *shape]: the padding rows of
+    # a fixed-size (graph) batch carry the slot index `slots`, which only this
+    # view holds, so whatever they write disturbs no request
+    state_padded: object = None
 
 
 class PageGroup:
@@ -62,7 +66,8 @@ class StateGroup:
     def __init__(self, spec: StateSpec):
         self.spec = spec
         self.layers: list[int] = []
-        self.tensor = None
+        self.tensor = None  # [layers, slots, *shape]
+        self.padded = None  # [layers, slots + 1, *shape], the same memory plus the spare slot
 
 
 class CacheManager:
@@ -138,10 +143,11 @@ class CacheManager:
                 dtype=dtype, device=device,
             )
         for g in self.state_groups:
-            g.tensor = torch.zeros(
-                len(g.layers), self.slots.num_slots, *g.spec.shape,
+            g.padded = torch.zeros(
+                len(g.layers), self.slots.num_slots + 1, *g.spec.shape,
                 dtype=getattr(torch, g.spec.dtype), device=device,
             )
+            g.tensor = g.padded[:, : self.slots.num_slots]
 
     def layer_cache(self, position: int, reader: bool = False) -> LayerCache:
         """The cache of schedule position `position`; `reader` marks a layer that
@@ -156,7 +162,8 @@ class CacheManager:
                 window=g.spec.window,
             )
         g = self.state_groups[gi]
-        return LayerCache(group=gi, owned=not reader, state=None if g.tensor is None else g.tensor[li])
+        return LayerCache(group=gi, owned=not reader, state=None if g.tensor is None else g.tensor[li],
+                          state_padded=None if g.padded is None else g.padded[li])
 
     def owns_cache(self, position: int) -> bool:
         return position in self._where

@@ -79,6 +79,22 @@ class BlockSpec:
 
 
 @dataclass(frozen=True)
+class TokenEmbeddingSpec:
+    """x = table[token id], no scaling."""
+
+    kind: ClassVar[str] = "token_lookup"
+    vocab_size: int
+
+
+@dataclass(frozen=True)
+class LinearHeadSpec:
+    """logits = x @ W.T, no bias."""
+
+    kind: ClassVar[str] = "linear"
+    vocab_size: int
+
+
+@dataclass(frozen=True)
 class ScheduleEntry:
     """One run of a block.  ``cache_of`` names an earlier schedule position whose
     cache this run reads instead of owning one; None means it owns its cache."""
@@ -89,7 +105,11 @@ class ScheduleEntry:
 
 @dataclass(frozen=True)
 class ModelSpec:
-    """Token ids -> embedding -> schedule of blocks -> final norm -> output matrix."""
+    """Token ids -> embedding -> schedule of blocks -> final norm -> head.
+
+    ``embedding`` and ``head`` are part specs like the others; left as None they
+    are the plain table lookup and the plain output matrix over ``vocab_size``.
+    """
 
     architecture: str
     hidden_size: int
@@ -105,8 +125,14 @@ class ModelSpec:
     max_position_embeddings: int | None = None
     stored_dtype: str = "bfloat16"
     extra: dict = field(default_factory=dict, compare=False)
+    embedding: object = None
+    head: object = None
 
     def __post_init__(self):
+        if self.embedding is None:
+            object.__setattr__(self, "embedding", TokenEmbeddingSpec(self.vocab_size))
+        if self.head is None:
+            object.__setattr__(self, "head", LinearHeadSpec(self.vocab_size))
         if not self.schedule:
             object.__setattr__(
                 self, "schedule", tuple(ScheduleEntry(i) for i in range(len(self.blocks)))

@@ -12,26 +12,38 @@ first, then prompt portions, each sequence's tokens contiguous):
                                                sequence's first portion
   block_tables[g][S, blocks_g]                 page ids per page group
   out_rows[R]                                  rows whose logits are wanted
-  tile_seq[T]  tile_q0[T]                      prompt portions cut into tiles of 16
-                                               queries: sequence and first query
+  extras[name]                                 int32 arrays that parts added in
+                                               their prepare() (launch lists of
+                                               their kernels and the like)
 
 The reference builds the same information per step as Python lists and one
 tensor per sequence (shrike/engine/model_runner.py:205-248).
+
+A step is described twice.  `StepShape` is the host's view before anything is
+on the device: the lengths, and what each part wants to add.  `StepContext` is
+what `forward` gets: the same numbers plus the device arrays.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass, field
 
+import numpy as np
 import torch
 
 
 class Workspace:
-    """Named device buffers that persist across steps and grow on demand."""
+    """Named device buffers that persist across steps and grow on demand.
 
-    def __init__(self, device):
+    `keep_outgrown`: a buffer that is replaced by a larger one stays allocated.
+    HIP graphs hold the addresses of the buffers they were recorded with; a
+    workspace that graphs share must never free one of them."""
+
+    def __init__(self, device, keep_outgrown: bool = False):
         self.device = device
+        self.keep_outgrown = keep_outgrown
         self._flat: dict[tuple[str, torch.dtype], torch.Tensor] = {}
+        self._outgrown: list[torch.Tensor] = []
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         numel = 1
@@ -40,9 +52,61 @@ class Workspace:
         key = (name, dtype)
         flat = self._flat.get(key)
         if flat is None or flat.numel() < numel:
+            if flat is not None and self.keep_outgrown:
+                self._outgrown.append(flat)
             flat = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._flat[key] = flat
         return flat[:numel].view(shape)
+
+    def nbytes(self) -> int:
+        held = list(self._flat.values()) + self._outgrown
+        return sum(t.numel() * t.element_size() for t in held)
+
+
+def bucket(n: int, floor: int = 1) -> int:
+    """The power of two (at least `floor`) that n rounds up to."""
+    b = floor
+    while b < n:
+        b *= 2
+    return b
+
+
+class StepShape:
+    """The host's description of a step before its metadata goes to the device.
+
+    The runner fills in the lengths; then every part's `prepare(shape)` may
+      * `add(name, array)`: an int32 array that travels with the step's one
+        metadata copy and comes back as `ctx.extras[name]` on the device;
+      * `notes[key] = value`: a decision taken on the host (a grid size, a
+        kernel variant) for its own `forward` to read from `ctx.notes`;
+      * `launch_key.append(x)`: anything hashable that its launches depend on
+        beyond the number of rows.  Steps are replayed from one HIP graph only
+        if their launch keys are equal.
+    Parts that share a key share the work: the first to prepare sets it, the
+    others find it there.  In a step of single tokens that is replayed from a
+    graph, what a part adds may depend on the step's shape only (row count and
+    launch key), never on its contents: the graph's later steps reuse it.
+    """
+
+    def __init__(self, q_lens: np.ndarray, starts: np.ndarray, page_size: int,
+                 padded_rows: int = 0):
+        self.q_lens = q_lens
+        self.starts = starts
+        self.ctx_lens = starts + q_lens
+        self.page_size = page_size
+        self.num_seqs = int(q_lens.size)
+        self.num_tokens = int(q_lens.sum())
+        self.num_decode = int((q_lens == 1).sum())  # sequences with one token come first
+        self.padded_rows = padded_rows  # trailing rows that stand for no request
+        self.max_decode_ctx = int(self.ctx_lens[: self.num_decode].max()) if self.num_decode else 0
+        self.extras: dict[str, np.ndarray] = {}
+        self.notes: dict = {}
+        self.launch_key: list = []
+
+    def add(self, name: str, array) -> None:
+        if name in self.extras:
+            raise KeyError(f"a part already added {name!r} to this step")
+        self.extras[name] = np.asarray(array, dtype=np.int64).reshape(-1)
 
 
 @dataclass
@@ -68,26 +132,9 @@ class StepContext:
     max_q_len: int = 0
     max_ctx_len: int = 0
     max_decode_ctx: int = 0  # longest context among the single-token sequences
-    tile_seq: torch.Tensor | None = None
-    tile_q0: torch.Tensor | None = None
-    num_prefill_tiles: int = 0
-
-    _wg_cache: dict = field(default_factory=dict)
+    # what the parts' prepare() added: device arrays, and host-side decisions
+    extras: dict = field(default_factory=dict)
+    notes: dict = field(default_factory=dict)
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)
-
-    def prefill_workgroups(self, tiles: int):
-        """Prompt portions cut into runs of `tiles` 16-query tiles: (sequence of
-        each run, its first query, number of runs), on the device."""
-        hit = self._wg_cache.get(tiles)
-        if hit is None:
-            seqs, q0s = [], []
-            for s in range(self.num_decode, self.num_seqs):
-                for q0 in range(0, self.q_lens[s], 16 * tiles):
-                    seqs.append(s)
-                    q0s.append(q0)
-            both = torch.tensor([seqs, q0s], dtype=torch.int32).to(self.device)
-            hit = (both[0], both[1], len(seqs))
-            self._wg_cache[tiles] = hit
-        return hit

@@ -58,9 +58,12 @@ class LLMEngine:
             num_blocks = cfg.num_kv_blocks
         else:
             # shrike/engine/model_runner.py:165-174: a share of the free device memory
+            # ... less what the step function's own buffers will take, which do not
+            # exist yet: the pool must leave them room
+            reserve = workspace_reserve(model, runtime, cfg)
             free, _total = torch.cuda.mem_get_info(runtime.device)
             per_page = max(1, probe.bytes_per_page(elem))
-            num_blocks = max(1, int(free * cfg.gpu_mem_util) // per_page)
+            num_blocks = max(1, int(max(0, free - reserve) * cfg.gpu_mem_util) // per_page)
         self.cache = CacheManager(specs, cfg.block_size, num_blocks, max_slots=cfg.max_running,
                                   enable_prefix_caching=cfg.enable_prefix_caching)
         self.cache.allocate(runtime.dtype, runtime.device)
@@ -201,6 +204,31 @@ class LLMEngine:
                 cache.cache_hit_blocks / max(1, cache.cache_query_blocks), 3
             ),
         }
+
+
+def workspace_reserve(model, runtime, cfg: EngineConfig) -> int:
+    """Bytes of device memory that the step function's buffers take once serving
+    is under way, measured on a throwaway cache of a few pages: one step of the
+    largest batch of single tokens (all of them padding rows) and one of the
+    largest prompt portion.  Every batch bucket of the decode graphs has buffers
+    of its own, each half the next one's size, so the largest counts twice."""
+    from .runner import GRAPH_BATCH_BUCKETS, Workspace
+
+    pages = -(-cfg.max_tokens_per_step // cfg.block_size) + 1
+    cache = CacheManager(model.cache_specs(), cfg.block_size, pages, max_slots=2,
+                         enable_prefix_caching=False)
+    cache.allocate(runtime.dtype, runtime.device)
+    runner = ModelRunner(model, cache, runtime, graphs=False)
+    rows = min(cfg.max_running, cfg.max_tokens_per_step, GRAPH_BATCH_BUCKETS[-1])
+    rows = next(b for b in GRAPH_BATCH_BUCKETS if b >= rows)
+    sizes = []
+    for singles, portion in ((rows, 0), (0, cfg.max_tokens_per_step)):
+        runner.workspace = Workspace(runtime.device)
+        runner.dry_run(singles, portion)
+        sizes.append(runner.workspace.nbytes())
+    torch.cuda.synchronize(runtime.device)
+    slack = 64 << 20  # graph objects, pinned staging, the sampler's scratch
+    return 2 * sizes[0] + sizes[1] + slack
 
 
 class LLM:

@@ -12,17 +12,18 @@ short kernels whose launches would otherwise cost more than they run.
 
 from __future__ import annotations
 
+from collections import OrderedDict
 from dataclasses import dataclass
 
 import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, SequenceCache
-from .context import StepContext, Workspace
-from .runtime import bucket
+from .context import StepContext, StepShape, Workspace
 
 GRAPH_BATCH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 GRAPH_TABLE_QUANTUM = 64  # block-table widths of graphs are multiples of this
+MAX_GRAPHS = 24  # captured decode steps kept; the least recently used one goes first
 
 
 @dataclass
@@ -44,18 +45,22 @@ class _Meta:
     """The int32 metadata of a step, laid out in one buffer."""
 
     FIELDS = ("token_ids", "positions", "token_seq", "cu_q", "ctx_lens", "state_slots", "fresh",
-              "out_rows", "tile_seq", "tile_q0")
+              "out_rows")
 
-    def __init__(self, arrays: dict, tables: list[np.ndarray]):
+    def __init__(self, arrays: dict, tables: list[np.ndarray], shape: StepShape):
         self.arrays = arrays
         self.tables = tables
-        self.parts = [arrays[f] for f in self.FIELDS] + [t.reshape(-1) for t in tables]
+        self.shape = shape
+        self.extra_names = sorted(shape.extras)  # what the parts added in prepare()
+        self.names = list(self.FIELDS) + self.extra_names
+        self.parts = ([arrays[f] for f in self.FIELDS] + [shape.extras[n] for n in self.extra_names]
+                      + [t.reshape(-1) for t in tables])
         self.sizes = [int(p.size) for p in self.parts]
         self.total = int(sum(self.sizes))
 
     def views(self, dev: torch.Tensor, num_seqs: int) -> dict:
         out, off = {}, 0
-        for name, size in zip(self.FIELDS, self.sizes):
+        for name, size in zip(self.names, self.sizes):
             out[name] = dev[off : off + size]
             off += size
         tables = []
@@ -63,14 +68,15 @@ class _Meta:
             tables.append(dev[off : off + t.size].view(num_seqs, t.shape[1]))
             off += t.size
         out["block_tables"] = tables
+        out["extras"] = {n: out[n] for n in self.extra_names}
         return out
 
 
 class _DecodeGraph:
-    """A captured decode step for one (batch bucket, table widths, context bucket)."""
+    """A captured decode step for one (batch bucket, table widths, launch key)."""
 
-    def __init__(self, device):
-        self.workspace = Workspace(device)
+    def __init__(self, workspace: Workspace):
+        self.workspace = workspace  # shared by the graphs of one batch bucket
         self.graph = None
         self.meta_dev = None
         self.logits = None
@@ -100,11 +106,15 @@ class ModelRunner:
                 self.layer_caches.append(None)
         self._pinned = None
         self._pinned_free = None  # event: the last copy out of the pinned buffer is done
-        # Graphs replay fixed kernel arguments: a mixer that reads host-side
-        # metadata (state kept outside the kernels' view) cannot be captured.
-        self.use_graphs = bool(graphs) and not cache.state_groups and model.graph_safe()
-        self._graphs: dict[tuple, _DecodeGraph] = {}
+        # Graphs replay fixed kernel arguments: the model's parts say whether
+        # their launches can be recorded.
+        self.use_graphs = bool(graphs) and model.graph_safe()
+        self._graphs: OrderedDict[tuple, _DecodeGraph] = OrderedDict()
+        # one workspace per batch bucket, shared by its graphs: their buffers have
+        # the same shapes, and a buffer that one of them outgrows is kept
+        self._graph_workspaces: dict[int, Workspace] = {}
         self.graph_replays = 0
+        self.graph_captures = 0
 
     # ---------------------------------------------------------------- metadata
 
@@ -147,9 +157,9 @@ class ModelRunner:
         if pads:
             q_lens = np.concatenate([q_lens, np.ones(pads, dtype=np.int64)])
             starts = np.concatenate([starts, np.zeros(pads, dtype=np.int64)])
-        num_seqs = n_real + pads
-        num_tokens = int(q_lens.sum())
-        num_decode = int((q_lens == 1).sum())
+        shape = StepShape(q_lens, starts, self.cache.page_size, padded_rows=pads)
+        self.model.prepare(shape)
+        num_seqs, num_tokens, num_decode = shape.num_seqs, shape.num_tokens, shape.num_decode
         cu_q = np.zeros(num_seqs + 1, dtype=np.int64)
         np.cumsum(q_lens, out=cu_q[1:])
         token_seq = np.repeat(np.arange(num_seqs), q_lens)
@@ -168,8 +178,9 @@ class ModelRunner:
             out_rows = np.asarray(
                 [cu_q[slot_of[i]] + w for i, e in enumerate(entries) for w in e.want], dtype=np.int64
             )
-        state_slots = np.array([entries[i].cache.state_slot for i in order] + [0] * pads,
-                               dtype=np.int64)
+        # padding rows carry the spare slot, as they carry the spare page
+        state_slots = np.array([entries[i].cache.state_slot for i in order]
+                               + [self.cache.slots.num_slots] * pads, dtype=np.int64)
         fresh = np.array([int(entries[i].cache.fresh_state) for i in order] + [0] * pads,
                          dtype=np.int64)
         tables = []
@@ -182,16 +193,9 @@ class ModelRunner:
                 t[k, : len(row)] = row
             t[n_real:, :] = self.cache.num_pages  # the spare page
             tables.append(t)
-        # prompt portions in tiles of 16 queries for the MFMA attention kernel
-        tile_counts = -(-q_lens[num_decode:] // 16)
-        tile_seq = np.repeat(np.arange(num_decode, num_seqs), tile_counts)
-        tile_first = np.zeros(num_seqs - num_decode + 1, dtype=np.int64)
-        np.cumsum(tile_counts, out=tile_first[1:])
-        tile_q0 = (np.arange(int(tile_counts.sum())) - tile_first[tile_seq - num_decode]) * 16
         arrays = dict(token_ids=token_ids, positions=positions, token_seq=token_seq, cu_q=cu_q,
-                      ctx_lens=ctx_lens, state_slots=state_slots, fresh=fresh, out_rows=out_rows,
-                      tile_seq=tile_seq, tile_q0=tile_q0)
-        meta = _Meta(arrays, tables)
+                      ctx_lens=ctx_lens, state_slots=state_slots, fresh=fresh, out_rows=out_rows)
+        meta = _Meta(arrays, tables, shape)
         meta.q_lens, meta.ctx_lens = q_lens, ctx_lens
         meta.num_seqs, meta.num_tokens, meta.num_decode = num_seqs, num_tokens, num_decode
         return meta
@@ -207,8 +211,7 @@ class ModelRunner:
         dev.copy_(host, non_blocking=True)
         self._pinned_free.record()
 
-    def _context(self, meta: _Meta, dev: torch.Tensor, workspace: Workspace,
-                 max_decode_ctx: int | None = None) -> StepContext:
+    def _context(self, meta: _Meta, dev: torch.Tensor, workspace: Workspace) -> StepContext:
         v = meta.views(dev, meta.num_seqs)
         nd = meta.num_decode
         return StepContext(
@@ -216,14 +219,11 @@ class ModelRunner:
             num_tokens=meta.num_tokens, num_seqs=meta.num_seqs, num_decode=nd,
             token_ids=v["token_ids"], positions=v["positions"], token_seq=v["token_seq"],
             cu_q=v["cu_q"], ctx_lens=v["ctx_lens"], state_slots=v["state_slots"], fresh=v["fresh"],
-            out_rows=v["out_rows"], tile_seq=v["tile_seq"], tile_q0=v["tile_q0"],
-            num_prefill_tiles=int(meta.arrays["tile_seq"].size), block_tables=v["block_tables"],
+            out_rows=v["out_rows"], block_tables=v["block_tables"],
             q_lens=meta.q_lens.tolist(), ctx_lens_host=meta.ctx_lens.tolist(),
             max_q_len=int(meta.q_lens.max()), max_ctx_len=int(meta.ctx_lens.max()),
-            max_decode_ctx=(
-                max_decode_ctx if max_decode_ctx is not None
-                else (int(meta.ctx_lens[:nd].max()) if nd else 0)
-            ),
+            max_decode_ctx=int(meta.ctx_lens[:nd].max()) if nd else 0,
+            extras=v["extras"], notes=meta.shape.notes,
         )
 
     def build_context(self, entries: list[StepEntry]) -> StepContext:
@@ -249,24 +249,40 @@ class ModelRunner:
         for gi in range(len(self.cache.groups)):
             need = max(len(e.cache.tables[gi]) for e in entries)
             widths.append(-(-need // GRAPH_TABLE_QUANTUM) * GRAPH_TABLE_QUANTUM)
-        ctx_bucket = bucket(max(e.start + 1 for e in entries), 256)
-        return batch, tuple(widths), ctx_bucket
+        # what the parts' launches depend on beyond the number of rows (a mixer's
+        # split of long contexts, say): steps share a graph only if it is equal
+        starts = np.zeros(batch, dtype=np.int64)
+        starts[: len(entries)] = [e.start for e in entries]
+        shape = StepShape(np.ones(batch, dtype=np.int64), starts, self.cache.page_size,
+                          padded_rows=batch - len(entries))
+        self.model.prepare(shape)
+        return batch, tuple(widths), tuple(shape.launch_key)
 
     def _graph_step(self, entries: list[StepEntry], key) -> torch.Tensor:
-        batch, widths, ctx_bucket = key
+        batch, widths, _launch_key = key
         g = self._graphs.get(key)
+        if g is not None:
+            self._graphs.move_to_end(key)
         if g is None or not self._refresh(g, entries, widths):
             self._check(entries)
             order = list(range(len(entries)))
             meta = self._meta(entries, order, pad_to=batch, table_widths=list(widths))
             if g is None:
-                g = _DecodeGraph(self.runtime.device)
+                if len(self._graphs) >= MAX_GRAPHS:
+                    # the device may still be replaying the graph that goes
+                    torch.cuda.synchronize(self.runtime.device)
+                    self._graphs.popitem(last=False)
+                workspace = self._graph_workspaces.get(batch)
+                if workspace is None:
+                    workspace = Workspace(self.runtime.device, keep_outgrown=True)
+                    self._graph_workspaces[batch] = workspace
+                g = _DecodeGraph(workspace)
                 g.meta_dev = torch.zeros(meta.total, dtype=torch.int32, device=self.runtime.device)
                 g.pinned = torch.empty(meta.total, dtype=torch.int32, pin_memory=True)
                 g.host = g.pinned.numpy()
                 g.copied = torch.cuda.Event()
                 offsets, off = {}, 0
-                for name, size in zip(meta.FIELDS, meta.sizes):
+                for name, size in zip(meta.names, meta.sizes):
                     offsets[name] = off
                     off += size
                 offsets["tables"] = []
@@ -277,15 +293,21 @@ class ModelRunner:
                 self._fill(g, entries, meta)
                 g.meta_dev.copy_(g.pinned, non_blocking=True)  # the eager run below reads it
                 g.copied.record()
-                g.ctx = self._context(meta, g.meta_dev, g.workspace, max_decode_ctx=ctx_bucket)
-                # once eagerly: every workspace buffer exists before the capture starts
-                self.model.forward(g.ctx, self.layer_caches)
+                g.ctx = self._context(meta, g.meta_dev, g.workspace)
+                # This step itself runs kernel by kernel: every workspace buffer exists
+                # before the capture starts.  Recording executes nothing, so this
+                # run's logits are the step's result and the graph is not replayed
+                # now: a part that advances a state of its own must see each step once.
+                eager_logits = self.model.forward(g.ctx, self.layer_caches).clone()
                 torch.cuda.synchronize(self.runtime.device)
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
                     g.logits = self.model.forward(g.ctx, self.layer_caches)
                 g.graph = graph
                 self._graphs[key] = g
+                self.graph_captures += 1
+                self.graph_replays += 1  # counted with the steps that the graph path served
+                return eager_logits[: len(entries)]
             else:
                 self._fill(g, entries, meta)
         g.meta_dev.copy_(g.pinned, non_blocking=True)
@@ -373,6 +395,25 @@ class ModelRunner:
         for e in entries:
             e.cache.fresh_state = False
         return g.logits[:n]
+
+    def dry_run(self, singles: int, portion: int) -> None:
+        """Runs the model once on made-up tokens so that every buffer of such a
+        step exists: `singles` rows of one token, or else one sequence of
+        `portion` tokens.  The single-token rows are padding rows beside one
+        real row; the cache must be otherwise unused (its first pages are
+        written)."""
+        seq = self.cache.new_sequence()
+        try:
+            n = portion if not singles else 1
+            self.cache.append(seq, 0, n)
+            entries = [StepEntry(seq, [0] * n, 0, [n - 1])]
+            meta = self._meta(entries, [0], pad_to=singles)
+            dev = self.workspace.get("step_meta", (meta.total,), torch.int32)
+            self._upload(meta, dev)
+            self.model.forward(self._context(meta, dev, self.workspace), self.layer_caches)
+            torch.cuda.synchronize(self.runtime.device)
+        finally:
+            self.cache.free(seq)
 
     # -------------------------------------------------------------------- step
 

@@ -1,12 +1,11 @@
 """The runtime a model is loaded into: device, compute dtype, how matrices are
-held, and the choice of kernel for each matrix product and attention call.
+held, and the choice of kernel for each matrix product.
 
 float32: every product runs in the general float32 kernel (fused multiply-add,
-no matrix mode of reduced precision) and attention in the general kernel.
-bfloat16: weights are held in the MFMA operand layout; products with at most
-64 rows stream them once through the skinny MFMA kernel, larger ones run the
-LDS-staged MFMA kernel; attention runs on the MFMA kernels where the shapes
-allow, else in the general kernel.
+no matrix mode of reduced precision).  bfloat16: weights are held in the MFMA
+operand layout; products with at most 64 rows stream them once through the
+skinny MFMA kernel, larger ones run the LDS-staged MFMA kernel.  What a mixer
+does between its products is the mixer's own business.
 """
 
 from __future__ import annotations
@@ -82,60 +81,3 @@ class Runtime:
         out = ctx.buffer(name, (n, w.rows), self.dtype)
         self.linear(x, w, out, bias=bias)
         return out
-
-    def attend(self, ctx, qkv, out, spec, tables, cache) -> None:
-        """Attention of every token of the step over its sequence's cache."""
-        h, hkv, d = spec.num_heads, spec.num_kv_heads, spec.head_dim
-        q = qkv[:, : h * d]
-        if self.dtype == torch.bfloat16 and ops.attention_supports_mfma(
-            h, hkv, d, cache.page_size, qkv.stride(0)
-        ):
-            if ctx.num_decode:
-                nsplit = decode_splits(ctx.num_decode, hkv, ctx.max_decode_ctx)
-                partial = ctx.buffer("attn_partial", (ctx.num_decode * h * nsplit * (d + 2),),
-                                     torch.float32)
-                ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
-                                     cache.k_pool, cache.v_pool, cache.page_size, spec.window,
-                                     spec.scale, partial, nsplit)
-            tiles = ops.attention_prefill_shared_tiles(h, hkv, d) if ctx.num_prefill_tiles else 0
-            if tiles:
-                # few queries: smaller workgroups, so that there are enough for the chip
-                small = -(-ctx.num_prefill_tiles // tiles) * hkv < PREFILL_MIN_WORKGROUPS
-                if small and ops.attention_prefill_shared_tiles(h, hkv, d, small=True):
-                    tiles = ops.attention_prefill_shared_tiles(h, hkv, d, small=True)
-                else:
-                    small = False
-                wg_seq, wg_q0, count = ctx.prefill_workgroups(tiles)
-                ops.attention_prefill_shared(q, out, count, h, hkv, d, ctx.cu_q, ctx.ctx_lens, wg_seq,
-                                             wg_q0, tables, cache.k_pool, cache.v_pool,
-                                             cache.page_size, spec.window, spec.scale, small=small)
-            elif ctx.num_prefill_tiles:
-                ops.attention_prefill(q, out, ctx.num_prefill_tiles, h, hkv, d, ctx.cu_q,
-                                      ctx.ctx_lens, ctx.tile_seq, ctx.tile_q0, tables, cache.k_pool,
-                                      cache.v_pool, cache.page_size, spec.window, spec.scale)
-            return
-        ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.k_pool,
-                      cache.v_pool, cache.page_size, spec.window, spec.scale)
-
-
-# portions whose 16-wavefront workgroups would number fewer than this take 8-wavefront ones
-PREFILL_MIN_WORKGROUPS = 192
-
-
-def bucket(n: int, floor: int = 1) -> int:
-    """The power of two (at least `floor`) that n rounds up to."""
-    b = floor
-    while b < n:
-        b *= 2
-    return b
-
-
-def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
-    """Workgroups per (sequence, key/value head) of decode attention: enough to
-    put one on every compute unit (256), each with at least 256 keys for its
-    four wavefronts.  Both inputs are rounded up to powers of two first, so a
-    step gives the same result whether it runs kernel by kernel or as a graph
-    captured for its bucket."""
-    want = -(-256 // (bucket(num_seqs) * kv_heads))
-    most = max(1, bucket(max_ctx, 256) // 256)
-    return max(1, min(want, most, 64))

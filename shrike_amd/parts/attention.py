@@ -2,10 +2,62 @@
 
 from __future__ import annotations
 
+from dataclasses import dataclass
+
+import numpy as np
 import torch
 
 from ..kernels import ops
 from .base import Mixer, PagedKVSpec, ParamSpec, build_part, register_mixer
+
+QUERY_TILE = 16  # queries per tile of the MFMA kernels for prompt portions
+COMPUTE_UNITS = 256
+KEYS_PER_WORKGROUP = 256  # a decode workgroup's four wavefronts want at least this many keys
+MAX_KEY_SPLITS = 64
+# portions whose 16-wavefront workgroups would number fewer than this take 8-wavefront ones
+PREFILL_MIN_WORKGROUPS = 192
+
+
+def _pow2(n: int, floor: int = 1) -> int:
+    b = floor
+    while b < n:
+        b *= 2
+    return b
+
+
+def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
+    """Workgroups per (sequence, key/value head) of decode attention: enough to
+    put one on every compute unit, each with at least KEYS_PER_WORKGROUP keys
+    for its four wavefronts.  Both inputs are rounded up to powers of two first,
+    so a step gives the same result whether it runs kernel by kernel or as a
+    graph captured for a padded batch."""
+    want = -(-COMPUTE_UNITS // (_pow2(num_seqs) * kv_heads))
+    most = max(1, _pow2(max_ctx, KEYS_PER_WORKGROUP) // KEYS_PER_WORKGROUP)
+    return max(1, min(want, most, MAX_KEY_SPLITS))
+
+
+@dataclass
+class AttentionPlan:
+    """How one step's attention is launched for a (heads, kv heads, head size)."""
+
+    mfma: bool = False
+    nsplit: int = 1  # key splits of the single-token rows
+    kernel: str = ""  # for prompt portions: "shared", "tiles" or "" (none in the step)
+    small: bool = False  # "shared" with half as many wavefronts per workgroup
+    count: int = 0  # workgroups ("shared") or tiles ("tiles")
+    seq_name: str = ""  # names of the launch lists among the step's extras
+    q0_name: str = ""
+
+
+def portion_runs(q_lens, first_seq: int, run: int):
+    """Prompt portions cut into runs of `run` queries: (sequence of each run, its
+    first query within the portion)."""
+    counts = -(-np.asarray(q_lens, dtype=np.int64) // run)
+    seqs = np.repeat(np.arange(first_seq, first_seq + counts.size), counts)
+    first = np.zeros(counts.size + 1, dtype=np.int64)
+    np.cumsum(counts, out=first[1:])
+    q0 = (np.arange(int(counts.sum())) - first[seqs - first_seq]) * run
+    return seqs, q0
 
 
 class PagedAttention(Mixer):
@@ -77,7 +129,80 @@ class PagedAttention(Mixer):
             self.position.load(tensors, runtime)
         self.linear = runtime.linear
         self.linear_deferred = runtime.linear_deferred
-        self.attend = runtime.attend
+        self.dtype = runtime.dtype
+
+    # ------------------------------------------------------------ launch plans
+
+    @property
+    def plan_key(self):
+        s = self.spec
+        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim)
+
+    def prepare(self, shape) -> None:
+        """Decides once per step and head geometry how attention is launched:
+        the key splits of single-token rows, and for prompt portions the kernel
+        and its list of workgroups, which goes up with the step's metadata."""
+        key = self.plan_key
+        if key in shape.notes:
+            return  # a layer with the same geometry has prepared this step
+        s = self.spec
+        h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
+        plan = shape.notes[key] = AttentionPlan()
+        plan.mfma = self.dtype == torch.bfloat16 and ops.attention_supports_mfma(
+            h, hkv, d, shape.page_size, (h + 2 * hkv) * d)
+        if not plan.mfma:
+            return  # the general kernel takes every token alike
+        if shape.num_decode:
+            plan.nsplit = decode_splits(shape.num_decode, hkv, shape.max_decode_ctx)
+            shape.launch_key.append((key, plan.nsplit))
+        portions = shape.q_lens[shape.num_decode:]
+        if portions.size == 0:
+            return
+        tiles = ops.attention_prefill_shared_tiles(h, hkv, d)
+        if tiles:
+            plan.kernel = "shared"
+            num_tiles = int((-(-portions // QUERY_TILE)).sum())
+            small_tiles = ops.attention_prefill_shared_tiles(h, hkv, d, small=True)
+            # few queries: smaller workgroups, so that there are enough for the chip
+            if small_tiles and -(-num_tiles // tiles) * hkv < PREFILL_MIN_WORKGROUPS:
+                plan.small, tiles = True, small_tiles
+            seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE * tiles)
+        else:
+            plan.kernel = "tiles"
+            seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE)
+        plan.count = int(seqs.size)
+        plan.seq_name, plan.q0_name = f"attention_seq:{h}:{hkv}:{d}", f"attention_q0:{h}:{hkv}:{d}"
+        shape.add(plan.seq_name, seqs)
+        shape.add(plan.q0_name, q0)
+
+    def attend(self, ctx, qkv, out, tables, cache) -> None:
+        """Attention of every token of the step over its sequence's cache."""
+        s = self.spec
+        h, hkv, d = s.num_heads, s.num_kv_heads, s.head_dim
+        plan = ctx.notes.get(self.plan_key)
+        if plan is None:
+            raise RuntimeError(f"{self.name}: the step was not prepared for this mixer "
+                               "(the step function calls prepare() on every part)")
+        q = qkv[:, : h * d]
+        if not plan.mfma:
+            ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.k_pool,
+                          cache.v_pool, cache.page_size, s.window, s.scale)
+            return
+        if ctx.num_decode:
+            partial = ctx.buffer("attn_partial", (ctx.num_decode * h * plan.nsplit * (d + 2),),
+                                 torch.float32)
+            ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
+                                 cache.k_pool, cache.v_pool, cache.page_size, s.window, s.scale,
+                                 partial, plan.nsplit)
+        if plan.kernel == "shared":
+            ops.attention_prefill_shared(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
+                                         ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
+                                         cache.k_pool, cache.v_pool, cache.page_size, s.window,
+                                         s.scale, small=plan.small)
+        elif plan.kernel == "tiles":
+            ops.attention_prefill(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
+                                  ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
+                                  cache.k_pool, cache.v_pool, cache.page_size, s.window, s.scale)
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
         s = self.spec
@@ -104,7 +229,7 @@ class PagedAttention(Mixer):
             write_kv=cache.owned, split_sum=split_sum,
         )
         attn = ctx.buffer("attn_out", (n, s.num_heads * s.head_dim), ctx.dtype)
-        self.attend(ctx, qkv, attn, s, tables, cache)
+        self.attend(ctx, qkv, attn, tables, cache)
         # the norm that follows adds the output to the residual stream and can add up parts
         return self.linear_deferred(ctx, "attn_proj", attn, self.w_o, bias=self.b_o)
 

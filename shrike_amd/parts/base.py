@@ -14,6 +14,13 @@ width; it never sees which model it is in.  It declares the tensors it needs
 * FeedForward:       forward(ctx, x) -> [N, width]; token by token.
 * Block:             forward(ctx, hidden, cache) ; arranges norms, mixer and
                      feed-forward around the residual stream.
+* Embedding:         forward(ctx) -> float32 [N, width], the residual stream's
+                     first value, from ctx.token_ids (and ctx.positions).
+* Head:              forward(ctx, x) -> float32 [R, vocab] from the normed rows.
+
+Any part may implement prepare(shape): it is called once per step, before the
+step's metadata goes to the device, with the host-side StepShape; there a part
+decides how its kernels will be launched and adds the index arrays they need.
 
 To add a part: write its spec dataclass with a unique ``kind``, write the
 class, and register it with the matching ``register_*`` function.
@@ -31,8 +38,9 @@ import torch
 class ParamSpec:
     """One tensor a part needs from the weight file.
 
-    init: how the random-weights mode draws it: "matrix" and "bias" are
-        N(0, 0.02), "norm" is 1 + N(0, 0.1).
+    init: how the random-weights mode draws it: "matrix", "embedding" and
+        "bias" are N(0, 0.02), "norm" is 1 + N(0, 0.1); the "unit" mode scales
+        a "matrix" by its fan-in and leaves an "embedding" at N(0, 1).
     keep_float32: held in float32 whatever the compute dtype (vectors that
         enter float32 arithmetic); others are held in the compute dtype.
     """
@@ -96,6 +104,11 @@ class Part:
     def check(self, runtime) -> None:
         """Raise if the kernels cannot take this part's sizes."""
 
+    def prepare(self, shape) -> None:
+        """Called once per step with the host-side StepShape, before anything is
+        copied to the device: decide launches, `shape.add` index arrays,
+        leave `shape.notes` for forward, extend `shape.launch_key`."""
+
 
 class Norm(Part):
     def forward(self, ctx, hidden: HiddenState, rows=None, write_resid=True) -> torch.Tensor:
@@ -114,6 +127,12 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # A mixer whose cache is a StateSpec is recorded into HIP graphs only if it
+    # says that its forward finds its state through ctx.state_slots and
+    # ctx.fresh on the device (nothing read on the host, no launch that depends
+    # on which slots the step uses).
+    state_graph_safe = False
+
     def cache_spec(self):
         """PagedKVSpec, StateSpec or None."""
         return None
@@ -134,12 +153,34 @@ class Block(Part):
         raise NotImplementedError
 
 
+class Embedding(Part):
+    """Built from a spec with `vocab_size`; `table` is what a tied head may share."""
+
+    table: torch.Tensor | None = None
+
+    def forward(self, ctx) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Head(Part):
+    """Logits from the normed rows.  `tie(embedding)` is called before load when
+    the model ties its output matrix to the embedding."""
+
+    def tie(self, embedding: Embedding) -> None:
+        raise NotImplementedError
+
+    def forward(self, ctx, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
 _REGISTRIES: dict[str, dict[str, Callable]] = {
     "norm": {},
     "position": {},
     "mixer": {},
     "ffn": {},
     "block": {},
+    "embedding": {},
+    "head": {},
 }
 
 
@@ -165,6 +206,14 @@ def register_ffn(kind: str, cls) -> None:
 
 def register_block(kind: str, cls) -> None:
     _register("block", kind, cls)
+
+
+def register_embedding(kind: str, cls) -> None:
+    _register("embedding", kind, cls)
+
+
+def register_head(kind: str, cls) -> None:
+    _register("head", kind, cls)
 
 
 def build_part(family: str, spec, width: int, name: str):

@@ -8,6 +8,13 @@ Input, one JSON object a line on standard input:
 For a step in which something is wanted, OUT/<step>.f32 holds the logits at
 the wanted places, in the order of the entries and of `want`, as little-endian
 float32 [wanted, vocab].  After every step a line `done <step>` is printed.
+
+--poison fills every cache page with NaN before the first step, and again each
+page that a request gives back (at its end, or when a window has passed it):
+a read through a stale table or beyond a request's length then shows as NaN.
+--pages writes OUT/<step>.pages.json: for each entry of the step the page ids
+of its block tables (one list per page group, -1 for a page given back) and
+the pages this step's tokens were written to.
 """
 
 from __future__ import annotations
@@ -31,6 +38,9 @@ def main(argv=None) -> int:
                     help="most tokens live requests hold at any time (each rounded up to 64)")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--no-graphs", action="store_true", help="launch every step kernel by kernel")
+    ap.add_argument("--poison", action="store_true",
+                    help="fill pages that no request holds with NaN (at start and when given back)")
+    ap.add_argument("--pages", action="store_true", help="write <step>.pages.json with the page ids used")
     args = ap.parse_args(argv)
 
     out_dir = Path(args.out)
@@ -46,6 +56,7 @@ def main(argv=None) -> int:
     from ..cache import CacheManager
     from ..engine.loading import load_model
     from ..engine.runner import ModelRunner, StepEntry
+    from .poison import PagePoisoner
 
     _say(f"loading {args.model} as {args.dtype}")
     model, runtime, _cfg = load_model(args.model, args.dtype)
@@ -55,7 +66,10 @@ def main(argv=None) -> int:
                          enable_prefix_caching=False)
     cache.allocate(runtime.dtype, runtime.device)
     runner = ModelRunner(model, cache, runtime, graphs=not args.no_graphs)
-    _say(f"ready: {num_pages} pages of {page} tokens")
+    poisoner = PagePoisoner(cache) if args.poison else None
+    if poisoner is not None:
+        poisoner.poison_everything()
+    _say(f"ready: {num_pages} pages of {page} tokens" + (", poisoned" if poisoner else ""))
 
     live: dict[str, tuple] = {}  # id -> (SequenceCache, tokens so far)
     for line in sys.stdin:
@@ -64,7 +78,7 @@ def main(argv=None) -> int:
             continue
         msg = json.loads(line)
         step = msg["step"]
-        entries, lengths = [], []
+        entries, lengths, used = [], [], []
         for e in msg.get("entries", []):
             rid = str(e["id"])
             if rid not in live:
@@ -82,6 +96,12 @@ def main(argv=None) -> int:
             entries.append(StepEntry(seq, tokens, have, [int(w) for w in e.get("want", [])]))
             live[rid][1] = have + len(tokens)
             lengths.append(have + len(tokens))
+            first, last = have // page, (have + len(tokens) - 1) // page
+            used.append({"id": rid, "start": have, "tokens": len(tokens),
+                         "tables": [list(t) for t in seq.tables],
+                         "written": [list(t[first : last + 1]) for t in seq.tables]})
+        if args.pages and entries:
+            (out_dir / f"{step}.pages.json").write_text(json.dumps(used) + "\n")
         if entries:
             logits = runner.step(entries)
             if logits.shape[0]:
@@ -90,11 +110,19 @@ def main(argv=None) -> int:
             else:
                 torch.cuda.synchronize()
             for e, length in zip(entries, lengths):
-                cache.trim(e.cache, length)
+                before = poisoner.held(e.cache) if poisoner else None
+                if cache.trim(e.cache, length) and poisoner:
+                    torch.cuda.synchronize()  # the step that still read them is done
+                    poisoner.poison_released(before, e.cache)
         for rid in msg.get("end", []):
             rid = str(rid)
             if rid in live:
-                cache.free(live.pop(rid)[0])
+                seq = live.pop(rid)[0]
+                before = poisoner.held(seq) if poisoner else None
+                cache.free(seq)
+                if poisoner:
+                    torch.cuda.synchronize()
+                    poisoner.poison_released(before)
         print(f"done {step}", flush=True)
     return 0
 

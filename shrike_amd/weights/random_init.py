@@ -19,7 +19,7 @@ from safetensors.torch import save_file
 
 from ..parts.base import ParamSpec
 
-_STD = {"matrix": 0.02, "bias": 0.02, "norm": 0.1}
+_STD = {"matrix": 0.02, "embedding": 0.02, "bias": 0.02, "norm": 0.1}
 
 #: "reference": the distributions above.  "unit": matrices N(0, 1/fan_in) (the
 #: embedding table N(0, 1)), biases N(0, 0.1): every part's output is as large
@@ -42,7 +42,9 @@ def random_tensor(p: ParamSpec, seed: int, dtype: torch.dtype, device="cpu",
         raise ValueError(f"{p.name}: unknown init {p.init!r}") from None
     if mode == "unit":
         if p.init == "matrix":
-            std = 1.0 if "embed" in p.name else float(p.shape[-1]) ** -0.5
+            std = float(p.shape[-1]) ** -0.5
+        elif p.init == "embedding":
+            std = 1.0
         elif p.init == "bias":
             std = 0.1
     elif mode != "reference":

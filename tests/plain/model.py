@@ -178,8 +178,10 @@ def decoder_layer(cfg: PlainConfig, w: dict, i: int, x, cos, sin):
     )
 
 
-def forward(cfg: PlainConfig, w: dict, token_ids: list[int], first_position: int = 0):
-    """Logits [N, V] of one whole sequence (qwen.py:160-164, 188-192).
+def forward(cfg: PlainConfig, w: dict, token_ids: list[int], first_position: int = 0, rows=None):
+    """Logits [N, V] of one whole sequence (qwen.py:160-164, 188-192); with
+    `rows`, of those positions only, selected after the final norm as the
+    reference does (qwen.py:190-191).
 
     Embedding lookup without scaling, the layers, the final norm, then the
     output matrix, which is the embedding table when the weights are tied and
@@ -194,6 +196,8 @@ def forward(cfg: PlainConfig, w: dict, token_ids: list[int], first_position: int
     for i in range(cfg.num_layers):
         x = decoder_layer(cfg, w, i, x, cos, sin)
     x = rms_norm(x, w["model.norm.weight"], cfg.rms_norm_eps)
+    if rows is not None:
+        x = x[torch.tensor(list(rows), dtype=torch.long)]
     head = w.get("lm_head.weight")
     if head is None:
         if not cfg.tie_word_embeddings:
@@ -209,8 +213,8 @@ class PlainModel:
         self.cfg = PlainConfig.from_dir(model_dir)
         self.weights = read_weights(model_dir, dtype)
 
-    def logits(self, token_ids: list[int]) -> torch.Tensor:
-        return forward(self.cfg, self.weights, list(token_ids))
+    def logits(self, token_ids: list[int], rows=None) -> torch.Tensor:
+        return forward(self.cfg, self.weights, list(token_ids), rows=rows)
 
     def greedy(self, prompt: list[int], max_new_tokens: int) -> list[int]:
         """Recompute the whole sequence for every new token; argmax takes the

@@ -252,3 +252,65 @@ def test_registration_continues_where_it_stopped():
     assert n == 3
     cm.free(seq)
     assert cm.match_prefix(cm.new_sequence(), tokens) == 12
+
+
+def test_poisoned_free_pages_show_through_a_shifted_table():
+    """The replay tool's poisoner on CPU tensors: keys written through a request's
+    own table read back finite; the same read through a table whose entry is
+    shifted to a free page, or to a page the request gave back, meets NaN."""
+    import torch
+
+    from shrike_amd.parts import PagedKVSpec
+    from shrike_amd.replay.poison import PagePoisoner
+
+    cache = CacheManager([PagedKVSpec(2, 32), PagedKVSpec(2, 32, window=8)], 4, 12, enable_prefix_caching=False)
+    cache.allocate(torch.float32, "cpu")
+    poisoner = PagePoisoner(cache)
+    poisoner.poison_everything()
+    assert all(torch.isnan(g.k_tensor).all() and torch.isnan(g.v_tensor).all() for g in cache.groups)
+
+    def write(seq, group, first, last):
+        g = cache.groups[group]
+        for p in range(first, last):
+            page = seq.tables[group][p // 4]
+            g.k_tensor[0, page, :, :, p % 4, :] = float(p)
+            g.v_tensor[0, page, :, :, p % 4] = float(p)
+
+    def read(table, group, first, last):
+        g = cache.groups[group]
+        return torch.stack([g.k_tensor[0, table[p // 4], :, :, p % 4, :].flatten() for p in range(first, last)])
+
+    a, b = cache.new_sequence(), cache.new_sequence()
+    cache.append(a, 0, 10)
+    cache.append(b, 0, 6)
+    for seq, n in ((a, 10), (b, 6)):
+        write(seq, 0, 0, n)
+        write(seq, 1, 0, n)
+    assert torch.isfinite(read(a.tables[0], 0, 0, 10)).all()
+    free_page = next(p for p in range(12) if cache.groups[0].pool.ref_count[p] == 0)
+    shifted = list(a.tables[0])
+    shifted[1] = free_page
+    assert torch.isnan(read(shifted, 0, 4, 8)).all()  # a stale entry reads poison, not old numbers
+    # the slots of a's last page beyond its 10 tokens were never written
+    assert torch.isnan(read(a.tables[0], 0, 10, 12)).all()
+
+    # the window passes a's first page: given back and poisoned, the others untouched
+    before = poisoner.held(a)
+    old_first = a.tables[1][0]
+    cache.append(a, 10, 2)
+    write(a, 0, 10, 12)
+    write(a, 1, 10, 12)
+    assert cache.trim(a, 12) == 1 and a.tables[1][0] == -1
+    assert poisoner.poison_released(before, a) == [[], [old_first]]
+    assert torch.isnan(cache.groups[1].k_tensor[0, old_first]).all()
+    assert torch.isfinite(read(a.tables[1], 1, 5, 12)).all()
+
+    # b ends: its pages are poisoned, a's are not
+    before = poisoner.held(b)
+    cache.free(b)
+    assert poisoner.poison_released(before) == before
+    for gi, pages in enumerate(before):
+        assert torch.isnan(cache.groups[gi].v_tensor[0, pages]).all()
+    assert torch.isfinite(read(a.tables[0], 0, 0, 12)).all()
+    cache.free(a)
+    cache.check([])

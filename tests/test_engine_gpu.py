@@ -316,3 +316,107 @@ def test_random_arrivals_under_page_pressure_with_shared_prefixes(model_root):
             assert got[i] == want[i], f"request {i}"
     assert tight.cache.num_free == 22 and not tight.scheduler.running
     tight.cache.check([])
+
+
+def test_graph_cache_is_bounded_and_memory_stops_growing(model_root, monkeypatch):
+    """Decode steps over 3 batch buckets, contexts that change the split of the
+    keys three times, and two table widths, with room for 4 graphs only: graphs
+    are evicted and captured again, device memory stops growing after the first
+    pass, and every step's logits equal those of kernel-by-kernel execution."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine import runner as runner_module
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    monkeypatch.setattr(runner_module, "MAX_GRAPHS", 4)
+    model_dir = make_model_dir("B", model_root, dtype="bfloat16", mode="unit")
+    model, rt, cfg = load_model(model_dir, "bfloat16")
+    rng = random.Random(21)
+    work = []  # (batch, prompt length): 3 single-token steps follow each
+    for batch in (1, 3, 6):
+        for length in (250, 500, 1022):  # 1022 + 3 tokens: 65 pages, the wider table; 8 splits of the keys
+            work.append((batch, length, [[rng.randrange(cfg.vocab_size) for _ in range(length + 3)]
+                                         for _ in range(batch)]))
+
+    def one_pass(runner, cache):
+        outs = []
+        for batch, length, seqs_ids in work:
+            seqs = [cache.new_sequence() for _ in range(batch)]
+            for s, ids in zip(seqs, seqs_ids):
+                cache.append(s, 0, length)
+                runner.step([StepEntry(s, ids[:length], 0, [])])
+            for k in range(3):
+                entries = []
+                for s, ids in zip(seqs, seqs_ids):
+                    cache.append(s, length + k, 1)
+                    entries.append(StepEntry(s, [ids[length + k]], length + k, [0]))
+                outs.append(runner.step(entries).clone())
+            for s in seqs:
+                cache.free(s)
+        torch.cuda.synchronize()
+        return outs
+
+    def make(graphs):
+        cache = CacheManager(model.cache_specs(), 16, 6 * 65 + 2, enable_prefix_caching=False)
+        cache.allocate(rt.dtype, rt.device)
+        return ModelRunner(model, cache, rt, graphs=graphs), cache
+
+    eager_runner, eager_cache = make(False)
+    want = one_pass(eager_runner, eager_cache)
+    graph_runner, graph_cache = make(True)
+    first = one_pass(graph_runner, graph_cache)
+    after_first = torch.cuda.memory_allocated()
+    second = one_pass(graph_runner, graph_cache)
+    after_second = torch.cuda.memory_allocated()
+    assert graph_runner.graph_replays == 2 * 3 * len(work)
+    assert len(graph_runner._graphs) <= 4 < graph_runner.graph_captures  # graphs were evicted
+    assert len(graph_runner._graph_workspaces) == 3  # one set of buffers per batch bucket
+    for a, b, c in zip(want, first, second):
+        assert torch.equal(a, b) and torch.equal(a, c)
+    # the second pass captures again what was evicted, into the buffers that exist
+    assert after_second - after_first <= 1 << 20
+    held = sum(w.nbytes() for w in graph_runner._graph_workspaces.values())
+    assert held <= 8 * 6 * (cfg.vocab_size * 4 + 64 * 1024)  # a few buffers of [rows, vocab] at most
+
+
+def test_bfloat16_generation_survives_preemption(model_root):
+    """Pages run out in bfloat16 too: preempted requests recompute in portions
+    and every token is the plain model's choice, or differs from it only where
+    the plain model's two best logits nearly tie (tests/test_paged.py:88-99)."""
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+
+    model_dir = make_model_dir("A", model_root, dtype="bfloat16", mode="unit")
+    plain = PlainModel(model_dir)
+    prompts = prompts_for("A", [9, 14, 6, 11], seed=5)
+    tight = LLMEngine(str(model_dir), dtype="bfloat16", block_size=4, num_kv_blocks=12,
+                      max_tokens_per_step=7, enable_prefix_caching=False)
+    got = tight.generate(prompts, SamplingParams(max_new_tokens=20, ignore_eos=True))
+    assert tight.metrics()["preemptions"] > 0
+    for prompt, out in zip(prompts, got):
+        assert len(out) == 20
+        check_against_plain(plain, prompt, out, gap=0.05 * float(plain.logits(prompt).abs().max()))
+    assert tight.cache.num_free == 12 and not tight.has_work
+    tight.cache.check([])
+
+
+def test_pool_sized_from_free_memory_leaves_room_for_the_step_buffers(model_root):
+    from shrike_amd import SamplingParams
+    from shrike_amd.config import EngineConfig
+    from shrike_amd.engine.llm_engine import LLMEngine, workspace_reserve
+    from shrike_amd.engine.loading import load_model
+
+    model_dir = make_model_dir("B", model_root, dtype="bfloat16", mode="unit")
+    model, rt, _ = load_model(model_dir, "bfloat16")
+    cfg = EngineConfig(block_size=16, gpu_mem_util=0.001, max_tokens_per_step=300, max_running=40,
+                       dtype="bfloat16")
+    reserve = workspace_reserve(model, rt, cfg)
+    # at least: two sets of [64 rows, vocab] float32 logits, and the slack
+    assert reserve >= 2 * 64 * 503 * 4 + (64 << 20)
+    free, _ = torch.cuda.mem_get_info()
+    engine = LLMEngine(None, cfg, model=model, runtime=rt)
+    per_page = engine.cache.bytes_per_page(2)
+    assert engine.cache.num_pages <= int((free - reserve) * 0.001) // per_page + 1
+    assert engine.cache.num_pages >= int((free - reserve - (1 << 30)) * 0.001) // per_page
+    out = engine.generate([[5, 6, 7]], SamplingParams(max_new_tokens=4, ignore_eos=True))
+    assert len(out[0]) == 4

@@ -26,9 +26,16 @@ def dev(t, dtype=None):
 
 
 def close(got, want, dtype, scale=None):
+    """scale None: errors are measured against the largest wanted value.  With a
+    number: element by element against max(scale, |wanted|), since a stored value
+    cannot be closer to the truth than its format's spacing, which grows with the
+    value (bfloat16 values near 2.4 lie 0.0156 apart)."""
     want = want.double().cpu()
-    scale = want.abs().max().clamp_min(1e-30) if scale is None else scale
-    err = ((got.double().cpu() - want).abs().max() / scale).item()
+    if scale is None:
+        scale = want.abs().max().clamp_min(1e-30)
+    else:
+        scale = want.abs().clamp_min(scale)
+    err = ((got.double().cpu() - want).abs() / scale).max().item()
     assert err <= TOL[dtype], f"rel err {err:.3e} > {TOL[dtype]}"
 
 
@@ -476,7 +483,8 @@ def fill_pools(tables, k_pool, v_pool, ctx, page_size):
 @pytest.mark.parametrize(
     "heads, kv_heads, head_dim, page_size, window, nsplit",
     [(14, 2, 64, 16, None, 1), (14, 2, 64, 16, None, 5), (28, 4, 128, 16, None, 8), (6, 3, 96, 32, 40, 3),
-     (16, 1, 32, 64, None, 2), (5, 5, 256, 16, 100, 4), (8, 8, 160, 48, None, 64)],
+     (16, 1, 32, 64, None, 2), (5, 5, 256, 16, 100, 4), (8, 8, 160, 48, None, 64),
+     (40, 8, 128, 16, None, 1), (40, 8, 128, 16, None, 4)],  # five query heads per group
 )
 def test_attention_decode_mfma(ops, heads, kv_heads, head_dim, page_size, window, nsplit):
     """Context lengths of the reference's decode test (tests/test_triton_attention.py:40-42),
@@ -503,7 +511,8 @@ def test_attention_decode_mfma(ops, heads, kv_heads, head_dim, page_size, window
 
 @pytest.mark.parametrize(
     "heads, kv_heads, head_dim, page_size, window",
-    [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 256, 16, None)],
+    [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 256, 16, None),
+     (40, 8, 128, 16, None)],
 )
 def test_attention_prefill_mfma(ops, heads, kv_heads, head_dim, page_size, window):
     """Portions of 2 to 200 tokens, some with earlier context, tiles with fewer than 16 queries."""
@@ -642,7 +651,8 @@ def test_rope_kv_store_adds_up_a_split_product(ops, n, splits):
 @pytest.mark.parametrize(
     "heads, kv_heads, head_dim, page_size, window",
     [(14, 2, 64, 16, None), (28, 4, 128, 16, None), (6, 3, 96, 32, 40), (4, 1, 32, 64, 17), (5, 5, 128, 16, None),
-     (16, 2, 64, 16, 100), (3, 1, 128, 48, None), (16, 1, 32, 16, None), (12, 1, 64, 32, 50)],
+     (16, 2, 64, 16, 100), (3, 1, 128, 48, None), (16, 1, 32, 16, None), (12, 1, 64, 32, 50),
+     (40, 8, 128, 16, None)],
 )
 @pytest.mark.parametrize("small", [False, True])
 def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window, small):
@@ -685,3 +695,113 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
 def test_attention_prefill_shared_refuses_wide_groups(ops):
     assert ops.attention_prefill_shared_tiles(34, 2, 64) == 0  # 17 heads per group: the per-tile kernel serves it
     assert ops.attention_prefill_shared_tiles(8, 2, 256) == 0
+
+
+def fill_pools_from(tables, k_pool, v_pool, seq, keys, values, page_size):
+    """Whole sequences of keys/values [ctx, kv_heads, head_dim] into sequence `seq`'s pages."""
+    ctx = keys.shape[0]
+    for first in range(0, ctx, page_size):
+        page = int(tables[seq, first // page_size])
+        n = min(page_size, ctx - first)
+        k = keys[first : first + n].to(k_pool.dtype).to(k_pool.device)  # [n, kv, d]
+        k_pool[page, :, :, :n, :] = k.view(n, k_pool.shape[1], k_pool.shape[2], k_pool.shape[4]).permute(1, 2, 0, 3)
+        v_pool[page, :, :, :n] = values[first : first + n].to(v_pool.dtype).to(v_pool.device).permute(1, 2, 0)
+
+
+@pytest.mark.parametrize("heads, kv_heads", [(28, 4), (40, 8)])
+@pytest.mark.parametrize("kernel", ["shared", "tiles"])
+def test_attention_prefill_over_two_thousand_keys(ops, heads, kv_heads, kernel):
+    """A 2,048-token prompt in one step (64 chunks of keys per query tile at the
+    end) beside a 300-token portion that starts at position 1,900.  Among random
+    scores near zero, chosen queries each have one key far away (or at a chunk's
+    or a page's edge) whose score stands out: a chunk of keys that is skipped,
+    read twice or masked wrongly changes those rows beyond the tolerance, where
+    uniform attention over thousands of keys would hide it."""
+    torch.manual_seed(31)
+    dtype = torch.bfloat16
+    head_dim, page_size, group = 128, 16, heads // kv_heads
+    seq_lens, starts = [2048, 300], [0, 1900]
+    ctx = [s + l for s, l in zip(starts, seq_lens)]
+    n = sum(seq_lens)
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, sum(-(-c // page_size) for c in ctx) + 3, kv_heads,
+                                         head_dim, dtype, seed=6)
+    q = torch.randn(n, heads, head_dim) * 0.3
+    keys = [torch.randn(c, kv_heads, head_dim) * 0.3 for c in ctx]
+    values = [torch.randn(c, kv_heads, head_dim) for c in ctx]
+    # (sequence, query position, key position): far back, the query's own key, edges of 32-key
+    # chunks and of pages, the first key of all
+    pairs = [(0, 2047, 0), (0, 2046, 2015), (0, 2040, 1000), (0, 1024, 1023), (0, 1025, 31), (0, 1026, 32),
+             (0, 16, 15), (0, 33, 0), (0, 15, 15), (0, 1500, 1471), (0, 777, 16), (0, 2031, 2031),
+             (1, 1900, 3), (1, 2199, 1899), (1, 2100, 1900), (1, 1915, 1915), (1, 2000, 63), (1, 2001, 64)]
+    amp = 20.0  # score of a pair: amp^2 / sqrt(128) = 35 against scores of a few units
+    for i, (s, p, j) in enumerate(pairs):
+        u = torch.zeros(head_dim)
+        u[(7 * i) % head_dim] = amp
+        row = sum(seq_lens[:s]) + p - starts[s]
+        head = (3 * i) % heads
+        q[row, head] = u
+        keys[s][j, head // group] = u
+    for s in range(2):
+        fill_pools_from(tables, k_pool, v_pool, s, keys[s], values[s], page_size)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
+    scale = head_dim**-0.5
+    qd = dev(q.to(dtype)).view(n, -1)
+    run = 16 * (ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim) if kernel == "shared" else 1)
+    wg_seq = [s for s, l in enumerate(seq_lens) for _ in range(0, l, run)]
+    wg_q0 = [q0 for l in seq_lens for q0 in range(0, l, run)]
+    args = (i32([0, 2048, n]), i32(ctx), i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, None, scale)
+    if kernel == "shared":
+        ops.attention_prefill_shared(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args)
+    else:
+        ops.attention_prefill(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args)
+    want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, seq_lens, starts, page_size, None, scale)
+    assert not torch.isnan(out.float()).any()
+    got = out.view(n, heads, head_dim)
+    close(got, want, dtype, scale=1.0)
+    for i, (s, p, j) in enumerate(pairs):  # each chosen row is its far key's value
+        row, head = sum(seq_lens[:s]) + p - starts[s], (3 * i) % heads
+        v = values[s][j, head // group].to(dtype).double()
+        assert (got[row, head].double().cpu() - v).abs().max() <= 2e-2 * v.abs().max(), (s, p, j)
+
+
+def test_attention_decode_finds_far_keys_in_a_long_context(ops):
+    """Single tokens at contexts up to 4,100 with the key splits the engine would
+    choose for them; every sequence has one key whose score stands out, at the
+    start, at a split's edge, at the very end."""
+    from shrike_amd.parts.attention import decode_splits
+
+    torch.manual_seed(32)
+    dtype = torch.bfloat16
+    heads, kv_heads, head_dim, page_size, group = 28, 4, 128, 16, 7
+    ctx = [4100, 4096, 2049, 2048, 1025, 300, 4097, 1]
+    special = [0, 4095, 1023, 2047, 512, 299, 2048, 0]
+    n = len(ctx)
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, sum(-(-c // page_size) for c in ctx) + 3, kv_heads,
+                                         head_dim, dtype, seed=7)
+    q = torch.randn(n, heads, head_dim) * 0.3
+    values = []
+    for s, c in enumerate(ctx):
+        keys, vals = torch.randn(c, kv_heads, head_dim) * 0.3, torch.randn(c, kv_heads, head_dim)
+        u = torch.zeros(head_dim)
+        u[(11 * s) % head_dim] = 20.0
+        q[s, (5 * s) % heads] = u
+        keys[special[s], ((5 * s) % heads) // group] = u
+        fill_pools_from(tables, k_pool, v_pool, s, keys, vals, page_size)
+        values.append(vals)
+    positions = torch.tensor([c - 1 for c in ctx], dtype=torch.int32)
+    scale = head_dim**-0.5
+    for nsplit in sorted({decode_splits(n, kv_heads, max(ctx)), decode_splits(1, kv_heads, max(ctx)), 1}):
+        out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
+        partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
+        ops.attention_decode(dev(q.to(dtype)).view(n, -1), out, n, heads, kv_heads, head_dim, dev(positions), tables,
+                             k_pool, v_pool, page_size, None, scale, partial, nsplit)
+        want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, [1] * n, [c - 1 for c in ctx],
+                                   page_size, None, scale)
+        got = out.view(n, heads, head_dim)
+        assert not torch.isnan(out.float()).any()
+        close(got, want, dtype, scale=1.0)
+        for s in range(n):
+            head = (5 * s) % heads
+            v = values[s][special[s], head // group].to(dtype).double()
+            assert (got[s, head].double().cpu() - v).abs().max() <= 2e-2 * v.abs().max(), (nsplit, s)

@@ -28,6 +28,12 @@ SHAPE = {
 }
 
 
+# One layer of the Qwen2.5-14B shape: 40 query heads over 8 key/value heads (groups
+# of 5), another width, another eps; a smaller vocabulary keeps the test short.
+SHAPE_14B = dict(SHAPE, hidden_size=5120, intermediate_size=13824, num_attention_heads=40,
+                 num_key_value_heads=8, rms_norm_eps=1e-5, vocab_size=32003)
+
+
 @pytest.fixture(scope="module")
 def model_dir(tmp_path_factory):
     from shrike_amd.weights import write_model_folder
@@ -36,21 +42,22 @@ def model_dir(tmp_path_factory):
 
 
 @pytest.fixture(scope="module")
-def reference(model_dir):
+def plain_model(model_dir):
+    return PlainModel(model_dir, dtype=torch.float32)  # float64 weights would not fit comfortably
+
+
+@pytest.fixture(scope="module")
+def reference(plain_model):
     rng = random.Random(5)
     ids = [rng.randrange(SHAPE["vocab_size"]) for _ in range(150)]
-    plain = PlainModel(model_dir, dtype=torch.float32)  # float64 weights would not fit comfortably
-    want = plain.logits(ids).double()
-    return ids, want
+    return ids, plain_model.logits(ids).double()
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
-def test_one_layer_of_the_7b_shape(dtype, tol, model_dir, reference):
+def four_cuttings(model_dir, dtype, tol, ids, want):
     from shrike_amd.cache import CacheManager
     from shrike_amd.engine.loading import load_model
     from shrike_amd.engine.runner import ModelRunner, StepEntry
 
-    ids, want = reference
     model, rt, _ = load_model(model_dir, dtype)
     cache = CacheManager(model.cache_specs(), 16, 24, enable_prefix_caching=False)
     cache.allocate(rt.dtype, rt.device)
@@ -90,8 +97,76 @@ def test_one_layer_of_the_7b_shape(dtype, tol, model_dir, reference):
     cache.check([])
 
 
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_one_layer_of_the_7b_shape(dtype, tol, model_dir, reference):
+    ids, want = reference
+    four_cuttings(model_dir, dtype, tol, ids, want)
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_one_layer_of_the_14b_shape(dtype, tol, tmp_path_factory):
+    """Five query heads per key/value head, width 5120: the four cuttings again."""
+    from shrike_amd.weights import write_model_folder
+
+    folder = tmp_path_factory.getbasetemp() / "big14"
+    if not (folder / "model.safetensors").is_file():
+        write_model_folder(dict(SHAPE_14B), folder, seed=9, mode="unit")
+    rng = random.Random(6)
+    ids = [rng.randrange(SHAPE_14B["vocab_size"]) for _ in range(150)]
+    want = PlainModel(folder, dtype=torch.float32).logits(ids).double()
+    four_cuttings(folder, dtype, tol, ids, want)
+
+
+@pytest.fixture(scope="module")
+def long_reference(plain_model):
+    """4,103 tokens through the plain model; logits at the rows the tests below ask for."""
+    rng = random.Random(8)
+    ids = [rng.randrange(SHAPE["vocab_size"]) for _ in range(4103)]
+    rows = [0, 15, 16, 1023, 2047] + list(range(4095, 4103))
+    return ids, plain_model.logits(ids, rows=rows).double()
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_a_2048_token_prompt_and_decoding_past_context_4096(dtype, tol, model_dir, long_reference):
+    """What the benchmark times, compared with the plain implementation: a
+    2,048-token prompt in one step (64 chunks of keys for the last query tile),
+    then the sequence grown to 4,095 tokens in portions, then 8 single tokens
+    through the graph path with the key splits the engine chooses itself."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    ids, want = long_reference
+    model, rt, _ = load_model(model_dir, dtype)
+    cache = CacheManager(model.cache_specs(), 16, 300, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    for g in cache.groups:  # a slot that is read before it is written shows up as NaN
+        g.k_tensor.fill_(float("nan"))
+        g.v_tensor.fill_(float("nan"))
+    runner = ModelRunner(model, cache, rt)
+    seq = cache.new_sequence()
+    cache.append(seq, 0, 2048)
+    first = runner.step([StepEntry(seq, ids[:2048], 0, [0, 15, 16, 1023, 2047])]).cpu().double()
+    assert rel_err(first, want[:5]) <= tol
+    p = 2048
+    for n in (1000, 512, 535):
+        cache.append(seq, p, n)
+        runner.step([StepEntry(seq, ids[p : p + n], p, [])])
+        p += n
+    assert p == 4095
+    rows = []
+    for p in range(4095, 4103):
+        cache.append(seq, p, 1)
+        rows.append(runner.step([StepEntry(seq, [ids[p]], p, [0])]).cpu().double()[0])
+    assert runner.graph_replays == 8
+    got = torch.stack(rows)
+    assert torch.isfinite(got).all()
+    assert rel_err(got, want[5:]) <= tol
+    cache.free(seq)
+
+
 @pytest.mark.parametrize("count", [100, 150])
-def test_many_single_tokens_as_a_graph_and_kernel_by_kernel(model_dir, count):
+def test_many_single_tokens_as_a_graph_and_kernel_by_kernel(model_dir, plain_model, count):
     """100 or 150 sequences decode together (graphs of 128 and 256 rows): a batch that the large product kernels
     serve (tiles of 128 and 256 tokens, operands loaded straight into LDS, shares
     of k).  Replayed from a HIP graph several times, with the program's own work
@@ -130,3 +205,9 @@ def test_many_single_tokens_as_a_graph_and_kernel_by_kernel(model_dir, count):
     eager, replayed = run(False), run(True)
     for a, b in zip(eager, replayed):
         assert torch.isfinite(a).all() and torch.equal(a, b)
+    # and both are right: some rows, the first and the last among them, against the
+    # plain implementation run on each sequence alone
+    for row in (0, 1, 37, 63, 64, count - 2, count - 1):
+        for step in (0, 3):
+            want = plain_model.logits(prompts[row] + feed[row][: step + 1], rows=[-1]).double()[0]
+            assert rel_err(replayed[step][row].cpu().double(), want) <= 3e-2, (row, step)

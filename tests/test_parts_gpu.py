@@ -448,3 +448,199 @@ def test_toy_position_encoding_through_the_unfused_path():
     want = want_for(ids)
     assert plain.rel_err(step_whole(runner, cache, ids), want) <= 1e-5
     assert plain.rel_err(step_whole(runner, cache, ids, [9] + [1] * 12), want) <= 1e-5
+
+
+# ---------------------- a toy state mixer that HIP graphs may record, with a prepare()
+
+
+@dataclass(frozen=True)
+class DeviceDecaySpec:
+    """The decay mixer again (s_t = decay * s_{t-1} + W x_t), computed on the device
+    from the step's own index arrays, so that decode steps replay from a graph."""
+
+    kind: ClassVar[str] = "toy_decay_device"
+    decay: float
+
+
+def define_graph_safe_state_mixer():
+    import numpy as np
+
+    from shrike_amd.parts import Mixer, ParamSpec, StateSpec, register_mixer
+
+    class DeviceDecayMixer(Mixer):
+        state_graph_safe = True  # the state is reached through ctx.state_slots on the device
+
+        def params(self):
+            return [ParamSpec(f"{self.name}.in_proj.weight", (self.width, self.width))]
+
+        def cache_spec(self):
+            return StateSpec((self.width,), "float32")
+
+        def load(self, tensors, runtime):
+            self.w = tensors[f"{self.name}.in_proj.weight"].float()
+
+        def prepare(self, shape):
+            """What forward needs beyond the step's common arrays: each token's
+            offset within its portion, and the last row of each sequence."""
+            if "decay_offset" in shape.extras:
+                return  # another layer of this kind has added them
+            first = np.cumsum(shape.q_lens) - shape.q_lens
+            shape.add("decay_offset", np.arange(shape.num_tokens) - np.repeat(first, shape.q_lens))
+            shape.add("decay_last_row", first + shape.q_lens - 1)
+            shape.notes["decay_prepared"] = shape.notes.get("decay_prepared", 0) + 1
+
+        def forward(self, ctx, x, cache):
+            u = x.float() @ self.w.t()  # [N, width]
+            n = u.shape[0]
+            seq, off = ctx.token_seq[:n].long(), ctx.extras["decay_offset"][:n].long()
+            slots = ctx.state_slots.long()
+            state = cache.state_padded  # padding rows of a graph batch use the spare slot
+            before = state[slots]  # [S, width], zero for a fresh slot
+            rows = torch.arange(n, device=u.device)
+            # y_t = sum_{j <= t, same sequence} decay^(t-j) u_j + decay^(offset+1) s_before
+            same = (seq[:, None] == seq[None, :]) & (rows[None, :] <= rows[:, None])
+            power = (rows[:, None] - rows[None, :]).clamp_min(0).float()
+            mix = torch.where(same, self.spec.decay ** power, torch.zeros_like(power))
+            y = mix @ u + (self.spec.decay ** (off.float() + 1))[:, None] * before[seq]
+            state.index_copy_(0, slots, y[ctx.extras["decay_last_row"].long()])
+            return y.to(x.dtype)
+
+    register_mixer("toy_decay_device", DeviceDecayMixer)
+
+
+def test_toy_state_mixer_with_prepare_is_replayed_from_graphs():
+    """A mixer with state of its own declares itself safe for graphs and adds its
+    own index arrays in prepare(): decode steps are captured and replayed, two
+    requests keep apart, and everything matches the recurrence computed plainly."""
+    from shrike_amd.engine.runner import StepEntry
+
+    define_graph_safe_state_mixer()
+    base = small_spec()
+    toy_block = replace(base.blocks[1], mixer=DeviceDecaySpec(decay=0.7), mixer_name="decay")
+    spec = replace(base, blocks=(base.blocks[0], toy_block))
+    w = cpu_weights(spec, seed=12)
+    runner, model, cache = make_runner(spec, w)
+    assert runner.use_graphs and model.graph_safe()
+
+    def want_for(ids):
+        cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
+        wd = {k: v.double() for k, v in w.items()}
+        n = len(ids)
+        cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+        x = plain.decoder_layer(cfg, wd, 0, wd["model.embed_tokens.weight"][torch.tensor(ids)], cos, sin)
+        p = "model.layers.1"
+        u = plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5) @ wd[f"{p}.decay.in_proj.weight"].t()
+        state, ys = torch.zeros(48, dtype=torch.float64), []
+        for t in range(n):
+            state = 0.7 * state + u[t]
+            ys.append(state)
+        x = x + torch.stack(ys)
+        h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
+        x = x + plain.swiglu(h, wd[f"{p}.mlp.gate_proj.weight"], wd[f"{p}.mlp.up_proj.weight"], wd[f"{p}.mlp.down_proj.weight"])
+        return plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+    g = torch.Generator().manual_seed(13)
+    a = torch.randint(0, 97, (40,), generator=g).tolist()
+    b = torch.randint(0, 97, (33,), generator=g).tolist()
+    wa, wb = want_for(a), want_for(b)
+    assert plain.rel_err(step_whole(runner, cache, a, [7, 2, 5] + [1] * 26), wa) <= 1e-5
+    replays = runner.graph_replays
+    assert replays == 26
+    # three requests decode side by side from one graph of four rows, each from its
+    # own slot; the fourth row is padding and writes to the spare slot only
+    sa, sb, sc = cache.new_sequence(), cache.new_sequence(), cache.new_sequence()
+    cache.append(sa, 0, 40)
+    cache.append(sb, 0, 33)
+    cache.append(sc, 0, 33)
+    runner.step([StepEntry(sa, a[:12], 0, []), StepEntry(sb, b[:5], 0, []), StepEntry(sc, b[:2], 0, [])])
+    for k in range(28):
+        out = runner.step([StepEntry(sa, [a[12 + k]], 12 + k, [0]), StepEntry(sb, [b[5 + k]], 5 + k, [0]),
+                           StepEntry(sc, [b[2 + k]], 2 + k, [0])]).cpu().double()
+        assert plain.rel_err(out, torch.stack([wa[12 + k], wb[5 + k], wb[2 + k]])) <= 1e-5
+    assert runner.graph_replays == replays + 28
+    for s in (sa, sb, sc):
+        cache.free(s)
+
+
+# ------------------------------------ a toy embedding and a toy head as parts of a model
+
+
+@dataclass(frozen=True)
+class ScaledEmbeddingSpec:
+    """x = multiplier * table[token] + position_table[position]."""
+
+    kind: ClassVar[str] = "toy_scaled_embedding"
+    vocab_size: int
+    multiplier: float
+    max_positions: int
+
+
+@dataclass(frozen=True)
+class CappedHeadSpec:
+    """logits = cap * tanh((x @ W.T) / cap)."""
+
+    kind: ClassVar[str] = "toy_capped_head"
+    vocab_size: int
+    cap: float
+
+
+def define_toy_embedding_and_head():
+    from shrike_amd.parts import Embedding, Head, ParamSpec, register_embedding, register_head
+
+    class ScaledEmbedding(Embedding):
+        def params(self):
+            return [ParamSpec(f"{self.name}.weight", (self.spec.vocab_size, self.width), init="embedding"),
+                    ParamSpec(f"{self.name}.positions", (self.spec.max_positions, self.width), init="embedding")]
+
+        def load(self, tensors, runtime):
+            self.table, self.positions = tensors[f"{self.name}.weight"], tensors[f"{self.name}.positions"]
+
+        def forward(self, ctx):
+            n = ctx.num_tokens
+            rows = self.table[ctx.token_ids[:n].long()].float() * self.spec.multiplier
+            return (rows + self.positions[ctx.positions[:n].long()].float()).contiguous()
+
+    class CappedHead(Head):
+        def tie(self, embedding):
+            self.tied_to = embedding
+
+        def params(self):
+            return [ParamSpec(f"{self.name}.weight", (self.spec.vocab_size, self.width), optional=True)]
+
+        def load(self, tensors, runtime):
+            w = tensors.get(f"{self.name}.weight")
+            self.w = (self.tied_to.table if w is None else w).float()
+
+        def forward(self, ctx, x):
+            return self.spec.cap * torch.tanh((x.float() @ self.w.t()) / self.spec.cap)
+
+    register_embedding("toy_scaled_embedding", ScaledEmbedding)
+    register_head("toy_capped_head", CappedHead)
+
+
+def test_toy_embedding_and_head_are_parts_like_the_others():
+    """An embedding with a multiplier and a learned position table, and a head that
+    caps its logits and shares the embedding's table: both come from the spec."""
+    define_toy_embedding_and_head()
+    base = small_spec()
+    spec = replace(base, embedding=ScaledEmbeddingSpec(97, 3.0, 64), head=CappedHeadSpec(97, 5.0),
+                   tie_word_embeddings=True)
+    w = cpu_weights(spec, seed=14)
+    assert "model.embed_tokens.positions" in w and "lm_head.weight" not in w
+    runner, model, cache = make_runner(spec, w)
+
+    def want_for(ids):
+        cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, True)
+        wd = {k: v.double() for k, v in w.items()}
+        n = len(ids)
+        cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+        x = 3.0 * wd["model.embed_tokens.weight"][torch.tensor(ids)] + wd["model.embed_tokens.positions"][:n]
+        for i in range(2):
+            x = plain.decoder_layer(cfg, wd, i, x, cos, sin)
+        x = plain.rms_norm(x, wd["model.norm.weight"], 1e-5)
+        return 5.0 * torch.tanh(plain.linear(x, wd["model.embed_tokens.weight"]) / 5.0)
+
+    ids = torch.randint(0, 97, (29,), generator=torch.Generator().manual_seed(15)).tolist()
+    want = want_for(ids)
+    assert plain.rel_err(step_whole(runner, cache, ids), want) <= 1e-5
+    assert plain.rel_err(step_whole(runner, cache, ids, [6, 1, 1, 2, 19]), want) <= 1e-5

@@ -37,7 +37,8 @@ def test_matrices_that_fill_the_chip_are_not_split():
 def test_key_splits_of_decode_attention_depend_on_the_buckets_only():
     """A graph is captured for a bucket of sequences and of context; every step
     that it replays must split the keys as the captured one did."""
-    from shrike_amd.engine.runtime import bucket, decode_splits
+    from shrike_amd.engine.context import bucket
+    from shrike_amd.parts.attention import decode_splits
 
     for kv_heads in (1, 4, 8):
         for seqs_lo, seqs_hi in ((1, 1), (3, 4), (5, 8), (33, 64), (129, 256)):
@@ -48,3 +49,50 @@ def test_key_splits_of_decode_attention_depend_on_the_buckets_only():
                 (n,) = plans
                 assert 1 <= n <= 64 and n <= max(1, bucket(ctx_hi, 256) // 256)
     assert decode_splits(8, 4, 2100) == 8 and decode_splits(64, 4, 4000) == 1 and decode_splits(1, 4, 100) == 1
+
+
+def test_decode_graphs_are_keyed_by_buckets_and_few():
+    """The key of a decode graph: batch bucket, table widths in steps of 64
+    pages, and what the parts' launches depend on (here the split of the keys).
+    Walking batch sizes and contexts far and wide makes a few dozen keys, not
+    one per context length."""
+    import numpy as np
+    import torch
+
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.config import AttentionSpec, BlockSpec, ModelSpec, RMSNormSpec, SwiGLUSpec
+    from shrike_amd.engine.runner import GRAPH_BATCH_BUCKETS, ModelRunner, StepEntry
+    from shrike_amd.engine.runtime import Runtime
+    from shrike_amd.models import DecoderModel
+
+    norm = RMSNormSpec(eps=1e-6)
+    mixer = AttentionSpec(num_heads=28, num_kv_heads=4, head_dim=128, qkv_bias=True, out_bias=False, scale=0.1)
+    block = BlockSpec(name="model.layers.0", mixer=mixer, ffn=SwiGLUSpec(intermediate_size=64),
+                      mixer_norm=norm, ffn_norm=norm)
+    model = DecoderModel(ModelSpec(architecture="t", hidden_size=3584, vocab_size=100, blocks=(block,),
+                                   final_norm=norm, tie_word_embeddings=False))
+    model.blocks[0].mixer.dtype = torch.bfloat16  # what load() would set
+    cache = CacheManager(model.cache_specs(), 16, 1 << 20)  # book-keeping only, nothing allocated
+    runner = ModelRunner(model, cache, Runtime("cuda:0", torch.bfloat16))
+    keys = {}
+    for batch in (1, 2, 3, 8, 9, 60, 64, 65, 200, 256):
+        seqs = [cache.new_sequence() for _ in range(batch)]
+        for ctx in (1, 100, 256, 257, 1000, 1024, 1025, 2047, 2049, 4000, 4097, 8000):
+            for s in seqs:
+                cache.append(s, 0, ctx)
+            entries = [StepEntry(s, [0], ctx - 1, [0]) for s in seqs]
+            key = runner._graph_key(entries)
+            assert key[0] == next(b for b in GRAPH_BATCH_BUCKETS if b >= batch)
+            assert key[1] == (-(-(-(-ctx // 16)) // 64) * 64,)
+            keys.setdefault(key, []).append((batch, ctx))
+        for s in seqs:
+            cache.free(s)
+    assert len(keys) <= 64  # of 120 (batch, context) pairs over 8 batch buckets and 6 table widths
+    # more than 256 rows, a portion, or a row that wants no logits: no graph
+    seqs = [cache.new_sequence() for _ in range(2)]
+    for s in seqs:
+        cache.append(s, 0, 8)
+    assert runner._graph_key([StepEntry(seqs[0], [0, 1], 0, [1])]) is None
+    assert runner._graph_key([StepEntry(seqs[0], [0], 0, [])]) is None
+    assert runner._graph_key([StepEntry(seqs[0], [0], 0, [0])] * 257) is None
+    assert np.all([len(v) >= 1 for v in keys.values()])

@@ -10,8 +10,9 @@ import pytest
 import torch
 
 from .plain.model import PlainModel
-from .tiny import CONFIGS, make_model_dir
-from .traces import TraceBuilder, changing_portions, last_one_by_one, mixed, run_trace, whole
+from .tiny import CONFIGS, PAGE_SIZES, make_model_dir
+from .traces import (TraceBuilder, changing_portions, check_pages, last_one_by_one, mixed, read_pages,
+                     run_trace, whole)
 
 pytestmark = pytest.mark.gpu
 
@@ -32,10 +33,16 @@ def model_root(tmp_path_factory):
     return tmp_path_factory.mktemp("models")
 
 
+# each tiny model at its own page size (4, 8, 16) and at 16, the size that serving uses
+CASES = sorted({(name, size) for name in "ABC" for size in (PAGE_SIZES[name], 16)})
+
+
 @pytest.mark.parametrize("mode", ["reference", "unit"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
-def test_four_cuttings_agree_with_the_plain_implementation(name, dtype, mode, model_root, tmp_path):
+@pytest.mark.parametrize("name, page_size", CASES)
+def test_four_cuttings_agree_with_the_plain_implementation(name, page_size, dtype, mode, model_root, tmp_path):
+    """Every free page is poisoned with NaN, at the start and whenever a request
+    gives it back: a row that read one would not pass the comparison."""
     model_dir = make_model_dir(name, model_root, dtype=dtype, mode=mode)
     vocab = CONFIGS[name]["vocab_size"]
     seqs = requests_for(name)
@@ -50,8 +57,12 @@ def test_four_cuttings_agree_with_the_plain_implementation(name, dtype, mode, mo
     # room for the largest request plus two small ones: the others wait for pages
     mixed_budget = budget + 128
     mixed(tb, "m_", seqs, mixed_budget, seed=3)
-    outputs = run_trace(model_dir, dtype, tb.steps, mixed_budget, tmp_path / "out", vocab)
+    outputs = run_trace(model_dir, dtype, tb.steps, mixed_budget, tmp_path / "out", vocab,
+                        block_size=page_size, poison=True, pages=True)
     got = tb.collect(outputs)
+    assert all(np.isfinite(rows).all() for rows in outputs.values())
+    reused = check_pages(tb.steps, read_pages(tmp_path / "out", tb.steps), page_size, mixed_budget // page_size)
+    assert reused > 0, "the pool was meant to be so small that pages are used again"
 
     scale = {rid: np.abs(w).max() for rid, w in want.items()}
     worst = {}
@@ -70,7 +81,7 @@ def test_four_cuttings_agree_with_the_plain_implementation(name, dtype, mode, mo
             cut, name_ = rid.split("_", 1)
             ref = got[(f"w_{name_}", pos)]
             assert np.abs(row - ref).max() / scale[name_] <= 1e-5
-    print(f"{name} {dtype} {mode}: worst rel err per cutting {worst}")
+    print(f"{name} page {page_size} {dtype} {mode}: worst rel err per cutting {worst}")
 
 
 def test_greedy_tokens_from_replayed_logits_match_plain(model_root, tmp_path):

@@ -17,14 +17,17 @@ TRACE_RUN = REPO / "bin" / "trace_run"
 
 
 def run_trace(model_dir, dtype: str, steps: list[dict], max_tokens: int, out_dir, vocab: int,
-              timeout: int = 600) -> dict[int, np.ndarray]:
+              timeout: int = 600, block_size: int | None = None, poison: bool = False,
+              pages: bool = False) -> dict[int, np.ndarray]:
     """-> {step: float32 [wanted, vocab]} for the steps that wanted something."""
     out_dir = Path(out_dir)
     out_dir.mkdir(parents=True, exist_ok=True)
     text = "".join(json.dumps(s) + "\n" for s in steps)
+    extra = ([] if block_size is None else ["--block-size", str(block_size)]) \
+        + (["--poison"] if poison else []) + (["--pages"] if pages else [])
     proc = subprocess.run(
         [sys.executable, str(TRACE_RUN), "--model", str(model_dir), "--dtype", dtype,
-         "--out", str(out_dir), "--max-tokens", str(max_tokens)],
+         "--out", str(out_dir), "--max-tokens", str(max_tokens), *extra],
         input=text, capture_output=True, text=True, timeout=timeout, env=dict(os.environ),
     )
     if proc.returncode != 0:
@@ -67,6 +70,56 @@ class TraceBuilder:
                 assert key not in got, f"{key} written twice"
                 got[key] = outputs[step][i]
         return got
+
+
+def read_pages(out_dir, steps: list[dict]) -> dict[int, list[dict]]:
+    """{step: what --pages wrote for it}."""
+    out = {}
+    for s in steps:
+        path = Path(out_dir) / f"{s['step']}.pages.json"
+        if path.exists():
+            out[s["step"]] = json.loads(path.read_text())
+    return out
+
+
+def check_pages(steps: list[dict], pages: dict[int, list[dict]], page_size: int, num_pages: int) -> int:
+    """What the page ids of a replay must satisfy: tables cover the tokens, ids lie
+    in the pool, no page is held by two live requests, and a request keeps its
+    pages from step to step.  Returns how many times a page was handed to a
+    request after another request had held it."""
+    reused = 0
+    groups = max((len(rec["tables"]) for recs in pages.values() for rec in recs), default=0)
+    for g in range(groups):
+        owner: dict[int, str] = {}  # page -> live request that holds it
+        seen_before: set[int] = set()
+        last_table: dict[str, list[int]] = {}
+        for s in steps:
+            for rec in pages.get(s["step"], []):
+                rid, table = rec["id"], rec["tables"][g]
+                assert len(table) * page_size >= rec["start"] + rec["tokens"]
+                assert all(-1 <= p < num_pages for p in table)
+                prev = last_table.get(rid, [])
+                assert all(a == b or b == -1 for a, b in zip(prev, table)), "a request's pages changed under it"
+                for a, b in zip(prev, table):  # given back by a window
+                    if a >= 0 and b == -1:
+                        seen_before.add(a)
+                        owner.pop(a, None)
+                for p in table[len(prev):]:
+                    if p == -1:
+                        continue  # taken and passed by the window within one step
+                    assert owner.get(p, rid) == rid, f"group {g}: page {p} is held twice"
+                    reused += p in seen_before
+                    owner[p] = rid
+                last_table[rid] = table
+                first = rec["start"] // page_size
+                written = rec["written"][g]
+                assert written == table[first : first + len(written)] and min(written) >= 0
+            for rid in s.get("end", []):
+                for p in last_table.pop(rid, []):
+                    if p >= 0:
+                        seen_before.add(p)
+                        owner.pop(p, None)
+    return reused
 
 
 def round64(n: int) -> int:
