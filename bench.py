@@ -8,10 +8,16 @@ The model has the layer sizes of the Qwen2.5-7B shape (28 layers, hidden 3584,
 152064) with random weights in bfloat16.  A "step" is one decode step of
 the whole serving path (LLMEngine.step: schedule, forward from the paged cache,
 sample, book-keeping) for `batch` requests that were each prefilled with 2,048
-random tokens; decoding runs towards context 4,096.  One JSON line is printed:
-`value` is decoded tokens per second; `prefill` is a 2,048-token prompt in one
-step; `roofline` prices the decode step's unavoidable HBM reads (every weight
-once, the live requests' cache) against 8 TB/s; `points` holds batch 1 and 64.
+random tokens; decoding runs towards context 4,096 (`--context N` starts it at
+N tokens instead).  One JSON line is printed: `value` is decoded tokens per
+second; `prefill` is a 2,048-token prompt in one step; `roofline` prices the
+decode step's unavoidable HBM reads (every weight once, the live requests'
+cache) against 8 TB/s, and against the bandwidth that a plain device copy
+reaches on this GPU (`achievable`); `prefill.achievable_frac` prices the prompt
+against the rate of the engine's own 4096^3 product; `points` holds batch 1 and
+64, and the same batches at a context near 4,000; `breakdown_us` is the decode
+step's time by kernel, from events around every launch of a step that runs
+kernel by kernel.
 """
 
 from __future__ import annotations
@@ -97,14 +103,16 @@ def make_engine(cfg, spec, max_batch: int, seed: int, budget: int | None = None)
     pages = max_batch * (CONTEXT_END // PAGE_SIZE + 2)
     config = EngineConfig(
         block_size=PAGE_SIZE, num_kv_blocks=pages,
-        max_tokens_per_step=budget if budget is not None else PROMPT_LEN + max_batch,
+        # a whole prompt, of any context this program asks for, beside every running request's token
+        max_tokens_per_step=budget if budget is not None else CONTEXT_END + max_batch,
         max_running=max_batch, enable_prefix_caching=False, dtype="bfloat16", seed=seed,
     )
     return LLMEngine(None, config, model=model, runtime=runtime)
 
 
-def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int) -> dict:
-    """Prefill `batch` prompts, then time `steps` decode steps."""
+def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int,
+               prompt_len: int = PROMPT_LEN) -> dict:
+    """Prefill `batch` prompts of `prompt_len` tokens, then time `steps` decode steps."""
     import torch
 
     from shrike_amd import SamplingParams
@@ -112,7 +120,7 @@ def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int) -> d
     rng = random.Random(seed)
     sampling = SamplingParams(max_new_tokens=batch + warmup + steps + 8, ignore_eos=True)
     for _ in range(batch):
-        engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)], sampling)
+        engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], sampling)
     while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
         engine.step()
     for _ in range(warmup):
@@ -160,6 +168,89 @@ def run_prefill(engine, cfg, seed: int, repeats: int = 3) -> dict:
     flops = prefill_flops(cfg, PROMPT_LEN)
     return {"value": round(PROMPT_LEN / best, 1), "tokens": PROMPT_LEN, "ms": round(best * 1e3, 3),
             "frac": round(flops / best / BF16_PEAK_FLOPS, 4)}
+
+
+def measure_peaks(device="cuda:0") -> dict:
+    """What this GPU reaches on the plainest work of each kind: bytes per second
+    of a device-to-device copy of 2 GiB (read + write), of a read-only pass (a
+    sum) over the same buffer, and flop/s of the engine's own bfloat16 product
+    at 4096 x 4096 x 4096."""
+    import torch
+
+    from shrike_amd.kernels import ops
+
+    out = {}
+    src = torch.empty(1 << 30, dtype=torch.bfloat16, device=device).normal_()
+    dst = torch.empty_like(src)
+
+    def timed(fn, repeats):
+        fn()
+        torch.cuda.synchronize()
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        for _ in range(repeats):
+            fn()
+        end.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(end) / repeats * 1e-3
+
+    nbytes = src.numel() * 2
+    out["copy_gbs"] = round(2 * nbytes / timed(lambda: dst.copy_(src), 5) / 1e9, 1)
+    out["read_gbs"] = round(nbytes / timed(lambda: src.view(torch.int16).max(), 5) / 1e9, 1)
+    del src, dst
+    n = 4096
+    a = torch.randn(n, n, device=device).to(torch.bfloat16)
+    wt = ops.retile_weight(torch.randn(n, n, device=device).to(torch.bfloat16))
+    c = torch.empty(n, n, dtype=torch.bfloat16, device=device)
+    out["gemm_tflops"] = round(2.0 * n**3 / timed(lambda: ops.gemm_tiled_weight(a, wt, n, n, c), 10) / 1e12, 1)
+    return out
+
+
+def kernel_breakdown(engine, steps: int = 3) -> dict:
+    """Microseconds per decode step by kernel: the running requests' next steps
+    run kernel by kernel (no graph) with an event before and after every launch."""
+    import torch
+
+    from shrike_amd.kernels import ops
+
+    names = ["embed", "add_rmsnorm", "silu_mul", "gemm", "gemm_tiled_weight", "rope_kv_store", "attention",
+             "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample"]
+    spans: list[tuple[str, object, object]] = []
+    saved = {n: getattr(ops, n) for n in names}
+
+    def wrap(name, fn):
+        def timed(*args, **kwargs):
+            label = name
+            if name == "gemm_tiled_weight":  # told apart by the matrix: [m, k]
+                label = f"gemm {args[2]}x{args[3]}" + (" gated" if kwargs.get("gated") else "")
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            out = fn(*args, **kwargs)
+            b.record()
+            spans.append((label, a, b))
+            return out
+        return timed
+
+    runner = engine.runner
+    graphs, runner.use_graphs = runner.use_graphs, False
+    engine._planned = None
+    try:
+        for n, fn in saved.items():
+            setattr(ops, n, wrap(n, fn))
+        engine.step()  # buffers of the kernel-by-kernel path
+        spans.clear()
+        for _ in range(steps):
+            engine.step()
+        torch.cuda.synchronize()
+    finally:
+        for n, fn in saved.items():
+            setattr(ops, n, fn)
+        runner.use_graphs = graphs
+        engine._planned = None
+    total: dict[str, float] = {}
+    for label, a, b in spans:
+        total[label] = total.get(label, 0.0) + a.elapsed_time(b) * 1e3 / steps
+    return {k: round(v, 1) for k, v in sorted(total.items(), key=lambda kv: -kv[1])}
 
 
 def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
@@ -213,6 +304,12 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=SHAPE_7B["num_hidden_layers"],
                     help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--context", type=int, default=PROMPT_LEN, metavar="N",
+                    help="start decoding at a context of N tokens (N-token prompts) instead of 2,048")
+    ap.add_argument("--far-context", type=int, default=4000 - 64, metavar="N",
+                    help="context of the extra points decode_b*_ctx4000 (0: leave them out)")
+    ap.add_argument("--no-peaks", action="store_true",
+                    help="skip the measurement of this GPU's copy bandwidth and product rate")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b",
                     help="layer sizes: Qwen2.5-7B (the default and the reported figure), 14B or 32B")
     ap.add_argument("--mixed", type=int, default=0, metavar="DECODES",
@@ -226,9 +323,12 @@ def main() -> int:
     if args.steps < 1 or args.warmup < 0 or args.batch < 1:
         print("bench.py: --steps and --batch must be positive, --warmup non-negative")
         return 2
-    room = CONTEXT_END - PROMPT_LEN - args.warmup - max(args.batch, 1 if args.no_points else 64) - 2
+    if not 1 <= args.context < CONTEXT_END:
+        print(f"bench.py: --context must lie in [1, {CONTEXT_END})")
+        return 2
+    room = CONTEXT_END - args.context - args.warmup - max(args.batch, 1 if args.no_points else 64) - 2
     if args.steps > room:
-        print(f"bench.py: at most {room} steps fit between the prompt and context {CONTEXT_END}")
+        print(f"bench.py: at most {room} steps fit between context {args.context} and {CONTEXT_END}")
         return 2
 
     import torch
@@ -261,17 +361,45 @@ def main() -> int:
 
     results = {}
     for b in batches:
-        results[b] = run_decode(engine, cfg, b, args.steps, args.warmup, args.seed + b)
+        results[b] = run_decode(engine, cfg, b, args.steps, args.warmup, args.seed + b, args.context)
         print(f"[bench] batch {b}: {results[b]['tok_s']:.1f} tok/s, "
               f"{results[b]['ms_per_step']:.3f} ms/step, {results[b]['gb_s']:.0f} GB/s",
               file=sys.stderr)
+    # the same batches near the end of the 4,096-token context, a short run each
+    far = {}
+    far_steps = min(args.steps, 40)
+    if args.far_context and not args.no_points and args.far_context + far_steps + args.warmup + 66 <= CONTEXT_END:
+        for b in batches:
+            far[b] = run_decode(engine, cfg, b, far_steps, args.warmup, args.seed + 100 + b, args.far_context)
+            print(f"[bench] batch {b} at context {far[b]['context_start']:.0f}: {far[b]['tok_s']:.1f} tok/s, "
+                  f"{far[b]['ms_per_step']:.3f} ms/step, {far[b]['gb_s']:.0f} GB/s", file=sys.stderr)
     prefill = run_prefill(engine, cfg, args.seed)
     print(f"[bench] prefill: {prefill}", file=sys.stderr)
+    # one batch left running for the per-kernel times
+    from shrike_amd import SamplingParams
+
+    rng = random.Random(args.seed + 7)
+    for _ in range(args.batch):
+        engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(args.context)],
+                           SamplingParams(max_new_tokens=64, ignore_eos=True))
+    while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
+        engine.step()
+    breakdown = kernel_breakdown(engine)
+    for req in list(engine.scheduler.running):
+        engine.abort(req.req_id)
+    print(f"[bench] decode step by kernel (us): {breakdown}", file=sys.stderr)
+    peaks = None if args.no_peaks else measure_peaks()
+    if peaks:
+        print(f"[bench] this GPU: {peaks}", file=sys.stderr)
+        prefill["gemm_tflops"] = peaks["gemm_tflops"]
+        prefill["achievable_frac"] = round(
+            prefill_flops(cfg, PROMPT_LEN) / (prefill["ms"] * 1e-3) / (peaks["gemm_tflops"] * 1e12), 4)
 
     main_run = results[args.batch]
     line = {
-        "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-{args.shape.upper()} shape, 2048-token prompts, "
-                  "decode to 4096)",
+        "metric": f"decode tok/s at batch {args.batch} (Qwen2.5-{args.shape.upper()} shape, "
+                  f"{args.context}-token prompts, decoding from context "
+                  f"{main_run['context_start']:.0f} to {main_run['context_end']:.0f})",
         "value": round(main_run["tok_s"], 1),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -295,7 +423,7 @@ def main() -> int:
             "vocab": cfg.vocab_size,
             "global_batch": args.batch,
             "seq_len": CONTEXT_END,
-            "prompt_len": PROMPT_LEN,
+            "prompt_len": args.context,
             "context_start": round(main_run["context_start"], 1),
             "context_end": round(main_run["context_end"], 1),
             "page_size": PAGE_SIZE,
@@ -312,8 +440,15 @@ def main() -> int:
             "frac": round(main_run["gb_s"] / HBM_PEAK_GBS, 4),
         },
         "points": {f"decode_b{b}": round(r["tok_s"], 1) for b, r in results.items() if b != args.batch},
+        "breakdown_us": breakdown,
     }
     line["points"][f"decode_b{args.batch}"] = round(main_run["tok_s"], 1)
+    for b, r in far.items():
+        line["points"][f"decode_b{b}_ctx4000"] = round(r["tok_s"], 1)
+    if peaks:
+        line["roofline"]["achievable"] = peaks["copy_gbs"]
+        line["roofline"]["achievable_read"] = peaks["read_gbs"]
+        line["roofline"]["achievable_frac"] = round(main_run["gb_s"] / max(peaks["copy_gbs"], peaks["read_gbs"]), 4)
     print(json.dumps(line))
     return 0
 

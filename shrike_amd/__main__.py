@@ -22,6 +22,9 @@ def parse_args(argv=None) -> argparse.Namespace:
     ap = argparse.ArgumentParser(prog="python -m shrike_amd", description=__doc__.split("\n\n")[0])
     ap.add_argument("prompt", nargs="?", default=None, help="text prompt (needs tokenizer.json)")
     ap.add_argument("--model", default=DEFAULT_MODEL_DIR)
+    ap.add_argument("--random-config", default=None, metavar="CONFIG_JSON",
+                    help="instead of --model: a config.json (or a folder with one) whose architecture "
+                         "is built with random weights drawn on the device from --seed")
     ap.add_argument("--prompt-ids", default=None, help="comma-separated token ids")
     ap.add_argument("--prompt-len", type=int, default=None, help="that many random token ids")
     ap.add_argument("--max-tokens", type=int, default=128)
@@ -46,12 +49,35 @@ def main(argv=None) -> int:
     from .engine.llm_engine import LLMEngine
 
     t0 = time.perf_counter()
-    engine = LLMEngine(
-        args.model, block_size=args.block_size, gpu_mem_util=args.gpu_mem_util,
+    options = dict(
+        block_size=args.block_size, gpu_mem_util=args.gpu_mem_util,
         max_tokens_per_step=args.max_tokens_per_step, max_running=args.max_running,
         enable_prefix_caching=not args.no_prefix_caching, num_kv_blocks=args.num_kv_blocks,
         dtype=args.dtype, seed=args.seed,
     )
+    if args.random_config is not None:
+        import json
+        import os
+
+        from .config import EngineConfig, architecture_name, canonical_dtype, get_architecture
+        from .engine.loading import random_model
+
+        path = args.random_config
+        if os.path.isdir(path):
+            path = os.path.join(path, "config.json")
+        try:
+            with open(path) as f:
+                raw = json.load(f)
+        except (OSError, ValueError) as e:
+            print(f"[error] --random-config {path}: {e}", file=sys.stderr)
+            return 2
+        arch = get_architecture(architecture_name(raw))
+        spec = arch.build_spec(arch.config_cls.from_dict(raw))
+        dtype = canonical_dtype(args.dtype) if args.dtype else spec.stored_dtype
+        model, runtime = random_model(spec, seed=args.seed, dtype=dtype)
+        engine = LLMEngine(None, EngineConfig(**dict(options, dtype=dtype)), model=model, runtime=runtime)
+    else:
+        engine = LLMEngine(args.model, **options)
     print(f"[engine up in {time.perf_counter() - t0:.1f}s, {engine.cache.num_pages} KV blocks]",
           file=sys.stderr)
     if args.prompt_ids is not None:

@@ -842,6 +842,223 @@ __global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per
                            accumulate, blockIdx.y);
 }
 
+
+// gemm_stream_kernel: for 17 to 64 tokens whose rows are 16-byte aligned with
+// k % 8 == 0.  Such a product is bound by the stream of weights, like the skinny
+// one, but its activations (up to 64 x k) are too many to fetch once per block of
+// weight rows.  What was measured on the chip shapes this kernel: a wavefront
+// pulls about 5 GB/s from memory however many loads it keeps in flight, and a
+// compute unit about 50 GB/s, so the stream needs 8 or more wavefronts on every
+// compute unit and the same work on each.  Hence one block of 16 weight rows per
+// wavefront (a gate block and its up block go to neighbouring wavefronts, which
+// combine their sums through LDS at the end), and workgroups of `waves` = 4 to 16
+// wavefronts, a number the host picks so that the launch is one workgroup for
+// each compute unit (or a whole number of rounds of them).
+//
+// k is walked in stages of kStreamTiles tiles.  Each wavefront streams its own
+// weight tiles straight into registers with non-temporal loads (nobody else needs
+// them); the stage's activations go from global memory straight into LDS in
+// units of whole cache lines, once for the workgroup: its NB * kStreamTiles units
+// are dealt out to the wavefronts, APER fetches each (where waves * APER exceeds
+// the units, some are fetched twice, into the same place).  Three stage buffers
+// and three sets of weight registers: while stage s is multiplied, the loads of
+// stages s + 1 and s + 2 are in flight, and one barrier per stage both publishes
+// a stage and frees the buffer of the stage before.  No load sits under a
+// condition: addresses are clamped into the matrices, tokens beyond n fill
+// output columns that are never written, columns beyond k meet the zeros that
+// pad the weight tiles, and tiles beyond the last one are not multiplied (only
+// the last stage of k can have such).  ksplit > 1 shares the stages among
+// workgroups, which leave float32 partial sums [ksplit][n][m] for the reading
+// kernel.
+constexpr int kStreamTiles = 4;
+
+template <int NB, int APER, bool GATED>
+__global__ void __launch_bounds__(16 * kWave)
+    gemm_stream_kernel(const bf16* __restrict__ a, int lda, int n, int k,
+                       const uint4* __restrict__ wt, int ktiles, int m,
+                       const float* __restrict__ bias, void* __restrict__ out, int ldo,
+                       int out_f32, int accumulate, int ksplit) {
+  constexpr int KT = kStreamTiles;
+  constexpr int kFrags = NB * KT;      // activation fragments per stage
+  constexpr int kLoads = APER + KT;    // loads per wavefront and stage
+  static_assert(2 * kLoads <= 63, "the load counter holds 63");
+  __shared__ u32x4 stage0[kFrags][kWave], stage1[kFrags][kWave], stage2[kFrags][kWave];
+  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
+  const int waves = blockDim.x / kWave;
+  const int j = lane % 16, kg = lane / 16;
+  // blocks of 16 weight rows; a gated weight has a gate and an up block per 16 output rows
+  const int wblocks = (GATED ? 2 : 1) * ((m + 15) / 16);
+  const int wb = blockIdx.x * waves + wave;  // this wavefront's block
+  const bool have_rows = wb < wblocks;
+  // a wavefront without rows streams the last block's weights; its sums are dropped
+  const u32x4* wrow = reinterpret_cast<const u32x4*>(wt) +
+                      static_cast<size_t>(have_rows ? wb : wblocks - 1) * ktiles * kWave + lane;
+
+  const int all_stages = (ktiles + KT - 1) / KT;
+  const int per = (all_stages + ksplit - 1) / ksplit;
+  const int st_first = blockIdx.y * per;
+  const int st_end = st_first + per < all_stages ? st_first + per : all_stages;
+  // the share's whole stages; the last stage of k may hold fewer than KT tiles
+  const int tail_tiles = (st_end == all_stages && ktiles % KT && st_first < st_end) ? ktiles % KT : 0;
+  const int full_end = tail_tiles ? st_end - 1 : st_end;
+
+  f32x4 acc[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) acc[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // What a wavefront fetches of the stage's activations, 1 KiB at a time: unit f is
+  // (token block f / KT, pair of tiles (f % KT) / 2, half of the block's tokens
+  // f % 2): 8 tokens x 128 bytes, lane l taking the 16 bytes at (token l % 8,
+  // chunk l / 8) - whole cache lines, where a fragment of 16 tokens x 64 bytes
+  // would use half of each line it touches.  In LDS the unit lies in lane order;
+  // lane (j, kg) of the operand of tile t finds its 16 bytes in unit (j / 8) at
+  // place j % 8 + 8 * (kg + 4 * (t % 2)): groups of 8 lanes read 128 contiguous
+  // bytes, without bank conflicts.  Beyond the last unit the first ones are
+  // fetched again.
+  static_assert(KT % 2 == 0, "tiles are fetched in pairs");
+  const bf16* asrc[APER];
+  int afrag[APER];
+#pragma unroll
+  for (int i = 0; i < APER; ++i) {
+    int f = wave + waves * i;
+    f = f < kFrags ? f : f % kFrags;
+    afrag[i] = f;
+    const int token = (f / KT) * 16 + (f % 2) * 8 + lane % 8;
+    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (lane / 8) * 8;
+  }
+  auto fetch = [&](u32x4 (&buf)[kFrags][kWave], u32x4 (&w)[KT], int st) {
+    // past the share's end: some stage that exists, never multiplied
+    int stage = st < all_stages ? st : all_stages - 1;
+    stage = stage < 0 ? 0 : stage;
+#pragma unroll
+    for (int i = 0; i < APER; ++i) {
+      const int col = (stage * KT + ((afrag[i] % KT) / 2) * 2) * 32;  // + (lane / 8) * 8 in asrc
+      SHK_LOAD_TO_LDS(asrc[i] + (col + (lane / 8) * 8 < k ? col : 0), &buf[afrag[i]][0]);
+    }
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+      const int tt = stage * KT + t;
+      w[t] = __builtin_nontemporal_load(wrow + static_cast<size_t>(tt < ktiles ? tt : ktiles - 1) * kWave);
+    }
+  };
+  const int xunit = j / 8, xplace = j % 8 + 8 * kg;  // where this lane's operands lie
+  auto multiply = [&](const u32x4 (&buf)[kFrags][kWave], const u32x4 (&w)[KT], int tiles) {
+#pragma unroll
+    for (int t = 0; t < KT; ++t) {
+      if (t < tiles) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b)
+          acc[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(bf16x8, w[t]),
+              __builtin_bit_cast(bf16x8, buf[b * KT + (t / 2) * 2 + xunit][xplace + 32 * (t % 2)]), acc[b],
+              0, 0, 0);
+      }
+    }
+  };
+  u32x4 w0[KT], w1[KT], w2[KT];
+  // Stage `now` has landed for every wavefront once each has waited for its own
+  // loads of it (the next stage's may stay in flight) and met the others; after
+  // the barrier nobody reads the stage before any more, so its buffer and its
+  // registers take the loads of the stage after next.
+#define SHK_STREAM_STEP(buf_now, w_now, buf_fill, w_fill, st_fill, tiles) \
+  SHK_WAIT_LOADS(kLoads);                                                  \
+  asm volatile("" ::: "memory");                                           \
+  __builtin_amdgcn_s_barrier();                                            \
+  asm volatile("" ::: "memory");                                           \
+  fetch(buf_fill, w_fill, st_fill);                                        \
+  __builtin_amdgcn_sched_barrier(0);                                       \
+  multiply(buf_now, w_now, tiles);
+  fetch(stage0, w0, st_first);
+  fetch(stage1, w1, st_first + 1);
+  int st = st_first;
+  for (; st + 3 <= full_end; st += 3) {
+    SHK_STREAM_STEP(stage0, w0, stage2, w2, st + 2, KT)
+    SHK_STREAM_STEP(stage1, w1, stage0, w0, st + 3, KT)
+    SHK_STREAM_STEP(stage2, w2, stage1, w1, st + 4, KT)
+  }
+  // up to two whole stages are left, and then the one that is not whole
+  const int left = full_end - st;
+  if (left >= 1) { SHK_STREAM_STEP(stage0, w0, stage2, w2, st + 2, KT) }
+  if (left >= 2) { SHK_STREAM_STEP(stage1, w1, stage0, w0, st + 3, KT) }
+  if (tail_tiles) {
+    if (left == 0) { SHK_STREAM_STEP(stage0, w0, stage2, w2, st + 2, tail_tiles) }
+    if (left == 1) { SHK_STREAM_STEP(stage1, w1, stage0, w0, st + 3, tail_tiles) }
+    if (left == 2) { SHK_STREAM_STEP(stage2, w2, stage1, w1, st + 4, tail_tiles) }
+  }
+#undef SHK_STREAM_STEP
+  SHK_WAIT_LOADS(0);  // no load may arrive in LDS that the workgroup has given back
+
+  int ob = wb;  // block of 16 output rows
+  if (GATED) {
+    // the wavefront of an up block hands its sums to its neighbour with the gate
+    // block, through the first stage buffer: room for the sums of kFrags / NB
+    // pairs at a time
+    f32x4* hand = reinterpret_cast<f32x4*>(&stage0[0][0]);
+    constexpr int kPairsPerPass = kFrags / NB;
+    const int pair = wave / 2;
+    for (int first = 0; first < waves / 2; first += kPairsPerPass) {
+      __syncthreads();  // the stage buffers, or the pass before, are read no more
+      const bool mine = pair >= first && pair < first + kPairsPerPass;
+      if (mine && (wave & 1)) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) hand[((pair - first) * NB + b) * kWave + lane] = acc[b];
+      }
+      __syncthreads();
+      if (mine && !(wave & 1)) {
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+          const f32x4 up = hand[((pair - first) * NB + b) * kWave + lane];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc[b][r] = silu(acc[b][r]) * up[r];
+        }
+      }
+    }
+    if (wave & 1) return;
+    ob = wb / 2;
+  }
+  if (!have_rows) return;
+
+  // lane (j, kg) of accumulator b: token b*16 + j, rows ob*16 + kg*4 + r
+  const int row0 = ob * 16 + kg * 4;
+#pragma unroll
+  for (int b = 0; b < NB; ++b) {
+    const int token = b * 16 + j;
+    if (token >= n || row0 >= m) continue;
+    float v[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      v[r] = acc[b][r];
+      if (bias && row0 + r < m) v[r] += bias[row0 + r];
+    }
+    if (ksplit > 1) {
+      float* o = static_cast<float*>(out) + (static_cast<size_t>(blockIdx.y) * n + token) * ldo + row0;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (row0 + r < m) o[r] = v[r];
+      continue;
+    }
+    const size_t idx = static_cast<size_t>(token) * ldo + row0;
+    if (out_f32) {
+      float* o = static_cast<float*>(out) + idx;
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+    } else {
+      bf16* o = static_cast<bf16*>(out) + idx;
+      if (row0 + 3 < m && (ldo & 3) == 0) {
+        uint2 packed;
+        packed.x = bf16_bits(v[0]) | (static_cast<uint32_t>(bf16_bits(v[1])) << 16);
+        packed.y = bf16_bits(v[2]) | (static_cast<uint32_t>(bf16_bits(v[3])) << 16);
+        *reinterpret_cast<uint2*>(o) = packed;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          if (row0 + r < m) o[r] = from_float<bf16>(v[r]);
+      }
+    }
+  }
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -1018,11 +1235,20 @@ extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   }
   if (mblocks >= 512) return 1;
   // up to 16 tokens: workgroups of 4 wavefronts share a block's k-tiles; more tokens:
-  // workgroups of 4 blocks walk k in stages of 4 tiles
-  int split = n <= 16 ? 8192 / (mblocks * 4) : 1024 / ((mblocks + 3) / 4);
-  const int most = ktiles / 16;
+  // every wavefront walks a block's k in stages of 4 tiles: about 2048 wavefronts
+  // fill the chip, but a share below 28 tiles is mostly start and end, and the
+  // reading kernel pays for every share (measured with 64 tokens, product and
+  // norm together: 3584 x 3584 16 us with 4 shares against 20 with 8; 3584 x
+  // 18944 37 us with 8 against 40 with 4)
+  int split, most;
+  if (n <= 16) {
+    split = 8192 / (mblocks * 4), most = ktiles / 16;
+    if (split > 16) split = 16;
+  } else {
+    split = 2048 / mblocks, most = ktiles / 28;
+    if (split > 8) split = 8;
+  }
   if (split > most) split = most;
-  if (split > 16) split = 16;
   return split > 1 ? split : 1;
 }
 
@@ -1066,6 +1292,43 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     else  // four wavefronts and two LDS buffers: two workgroups fit on a compute unit
       launch_big<2, 2, 4, 4, 2>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);
+    SHK_LAUNCH_CHECK("gemm_bf16");
+    return 0;
+  }
+  if (n > 16 && vec) {
+    // 17 to 64 tokens, aligned rows: every wavefront streams the weights of its own
+    // block of rows, the activations are shared through LDS.  Wavefronts per
+    // workgroup: so many that the launch is one workgroup for each of the 256
+    // compute units, or a whole number of rounds of them where 16 per workgroup
+    // do not suffice (an even number for gated weights: gate and up side by side).
+    const int wblocks = (gated ? 2 : 1) * mb;
+    const long long tasks = static_cast<long long>(wblocks) * ksplit;
+    // (more than a round's worth: workgroups of 8, two of which share a compute unit
+    // and fill each other's pauses)
+    int waves = tasks > 256 * 16 ? 8 : static_cast<int>((tasks + 255) / 256);
+    waves = waves < 4 ? 4 : waves;
+    if (gated) waves += waves & 1;
+    const int nb = n <= 32 ? 2 : 4;
+    const int aper = (nb * kStreamTiles + waves - 1) / waves;  // 1 to 4
+    dim3 sgrid((wblocks + waves - 1) / waves, ksplit);
+#define SHK_STREAM(NB, APER)                                                         \
+  do {                                                                               \
+    if (gated)                                                                       \
+      gemm_stream_kernel<NB, APER, true><<<sgrid, waves * kWave, 0, s>>>(            \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, ksplit);         \
+    else                                                                             \
+      gemm_stream_kernel<NB, APER, false><<<sgrid, waves * kWave, 0, s>>>(           \
+          ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, ksplit);         \
+  } while (0)
+    if (nb == 2) {
+      if (aper == 1) SHK_STREAM(2, 1); else SHK_STREAM(2, 2);
+    } else {
+      if (aper == 1) SHK_STREAM(4, 1);
+      else if (aper == 2) SHK_STREAM(4, 2);
+      else if (aper == 3) SHK_STREAM(4, 3);
+      else SHK_STREAM(4, 4);
+    }
+#undef SHK_STREAM
     SHK_LAUNCH_CHECK("gemm_bf16");
     return 0;
   }

@@ -420,3 +420,22 @@ def test_pool_sized_from_free_memory_leaves_room_for_the_step_buffers(model_root
     assert engine.cache.num_pages >= int((free - reserve - (1 << 30)) * 0.001) // per_page
     out = engine.generate([[5, 6, 7]], SamplingParams(max_new_tokens=4, ignore_eos=True))
     assert len(out[0]) == 4
+
+
+def test_command_line_builds_a_random_model_from_a_config(tmp_path, capsys):
+    """--random-config: no model folder, weights drawn on the device from the seed;
+    the same seed gives the same tokens, another seed gives others."""
+    import json
+
+    from shrike_amd.__main__ import main
+
+    path = tmp_path / "config.json"
+    path.write_text(json.dumps(dict(CONFIGS["B"], torch_dtype="bfloat16")))
+    runs = []
+    for seed in ("3", "3", "4"):
+        rc = main(["--random-config", str(path), "--prompt-len", "9", "--max-tokens", "6", "--seed", seed,
+                   "--num-kv-blocks", "16", "--ignore-eos"])
+        assert rc == 0
+        runs.append([int(t) for t in capsys.readouterr().out.split()])
+    assert len(runs[0]) == 6 and runs[0] == runs[1]
+    assert main(["--random-config", str(tmp_path / "absent.json"), "--prompt-len", "3"]) == 2

@@ -390,7 +390,11 @@ def test_sample_frequencies_follow_the_distribution(ops):
     [(1, 48, 64), (8, 3584, 3584), (7, 503, 128), (16, 100, 172), (17, 130, 96), (33, 200, 333),
      (48, 64, 64), (64, 1000, 520), (5, 37, 50), (65, 128, 64), (130, 200, 333), (300, 503, 128),
      (1000, 172, 96), (257, 130, 172), (2048, 1024, 512), (33, 200, 1600), (3, 48, 4000), (64, 100, 2100),
-     (40, 33000, 1000)],  # the last: 33 to 64 rows on the LDS-staged kernel
+     (40, 33000, 1000),
+     # 17 to 64 aligned rows: the kernel that streams weights per wavefront; whole and partial last
+     # stages of 128 of k, shares of k, fewer row blocks than a workgroup has wavefronts
+     (64, 3584, 3584), (64, 4608, 3584), (64, 3584, 18944), (17, 3584, 3584), (32, 100, 3584),
+     (33, 4608, 3616), (50, 72, 160), (24, 40, 32), (64, 66000, 96)],
 )
 def test_gemm_tiled_weight(ops, n, m, k):
     """The MFMA kernels over the tiled weight layout (weight-streaming up to 64
@@ -572,6 +576,7 @@ def test_attention_mfma_finds_one_far_key_among_thousands(ops):
 
 @pytest.mark.parametrize("n, inter, k", [(1, 172, 64), (8, 18944, 256), (20, 100, 96), (40, 352, 128), (64, 48, 50),
                                          (9, 100, 1700), (50, 64, 3000), (40, 16400, 1040),
+                                         (64, 18944, 3584), (17, 2000, 416), (32, 66000, 64),
                                          (65, 172, 64), (300, 1000, 520), (1000, 200, 96)])
 def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
     """One product over the interleaved gate/up weight yields silu(x g^T) * (x u^T)."""
@@ -587,7 +592,8 @@ def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
     close(out, want, dtype)
 
 
-@pytest.mark.parametrize("n, m, k", [(8, 3584, 3584), (1, 48, 4000), (33, 200, 1600), (64, 100, 2100),
+@pytest.mark.parametrize("n, m, k", [(8, 3584, 3584), (1, 48, 4000), (33, 200, 2400), (64, 100, 2100),
+                                     (64, 3584, 3584), (64, 4608, 3584), (64, 3584, 18944), (20, 3584, 18944),
                                      (100, 3584, 3584), (300, 136, 1100), (64, 2100, 16400), (40, 2100, 16400),
                                      (512, 5120, 5120)])  # the last: many tokens, tiles of 256 x 128 in three shares
 def test_split_product_and_its_readers(ops, n, m, k):
