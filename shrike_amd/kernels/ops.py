@@ -239,6 +239,9 @@ def rope_kv_store(qkv, heads, kv_heads, head_dim, rot_dim, inv_freq, positions, 
     n = qkv.shape[0]
     if not qkv.is_contiguous() or qkv.shape[1] != (heads + 2 * kv_heads) * head_dim:
         raise KernelError("rope_kv_store: qkv must be contiguous [n, (heads + 2 kv_heads) head_dim]")
+    # the kernel reads one position (and one sequence index) per row of qkv
+    if positions.shape[0] < n or (write_kv and token_seq.shape[0] < n):
+        raise KernelError(f"rope_kv_store: qkv has {n} rows but positions / token_seq are shorter")
     parts, splits, bias = None, 0, None
     if split_sum is not None:
         parts, bias = split_sum.parts, split_sum.bias

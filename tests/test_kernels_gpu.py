@@ -305,6 +305,17 @@ def test_attention_refuses_head_sizes_it_cannot_do(ops):
         ops.attention(z, torch.empty_like(z), 1, 1, 272, i, i, i.view(1, 1), k_pool, v_pool, 4, None, 1.0)
 
 
+def test_position_kernel_refuses_more_rows_than_positions(ops):
+    """Refused on the host: the kernel would read a position per row of qkv."""
+    from shrike_amd.kernels import KernelError
+
+    qkv = torch.zeros(5, 4 * 16, device="cuda")
+    i3 = torch.zeros(3, dtype=torch.int32, device="cuda")
+    k_pool, v_pool = torch.zeros(2, 1, 1, 4, 16, device="cuda"), torch.zeros(2, 1, 16, 4, device="cuda")
+    with pytest.raises(KernelError, match="positions"):
+        ops.rope_kv_store(qkv, 2, 1, 16, 0, None, i3, i3, i3.view(3, 1), k_pool, v_pool, 4)
+
+
 # ------------------------------------------------------------------- sampling
 
 
