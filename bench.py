@@ -240,6 +240,10 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
         engine.step()  # buffers of the kernel-by-kernel path
         spans.clear()
         for _ in range(steps):
+            # the device is held back while the host queues the step's launches and
+            # events, so that an event pair brackets its kernel and not the host's pace
+            torch.cuda.synchronize()
+            torch.cuda._sleep(30_000_000)
             engine.step()
         torch.cuda.synchronize()
     finally:
