@@ -761,18 +761,29 @@ __global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per
     const int block = mb0 + rb < mblocks ? mb0 + rb : mblocks - 1;
     wsrc[i] = wt + static_cast<size_t>(block) * ktiles * kWave + lane;
   }
+  // Activations, 1 KiB per load.  With stages of 64 of k (KS == 2) a load takes 8
+  // tokens x 128 bytes, lane l the 16 bytes at (token l % 8, chunk l / 8): whole cache
+  // lines, where a fragment of 16 tokens x 64 bytes uses half of each line it touches
+  // and asks the L2 twice as often.  Unit u holds tokens (u / 2) * 16 + (u % 2) * 8 ...
+  // in lane order; lane (j, kg) of the operand of step ks finds its 16 bytes in unit
+  // 2 * block + j / 8 at place j % 8 + 8 * (kg + 4 * ks): groups of 8 lanes read 128
+  // contiguous bytes, without bank conflicts.
+  constexpr bool kUnits = KS == 2;
 #pragma unroll
   for (int i = 0; i < kAPer; ++i) {
-    const int rb = (wave + kWaves * i) / KS;
-    const int token = tok0 + rb * 16 + lane % 16;
-    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (lane / 16) * 8;
+    const int f = wave + kWaves * i;
+    const int token = kUnits ? tok0 + (f / 2) * 16 + (f % 2) * 8 + lane % 8 : tok0 + (f / KS) * 16 + lane % 16;
+    asrc[i] = a + static_cast<size_t>(token < n ? token : n - 1) * lda + (kUnits ? lane / 8 : lane / 16) * 8;
   }
+  const int xunit = (lane % 16) / 8, xplace = lane % 8 + 8 * (lane / 16);
   auto load = [&](u32x4 (&buf)[kFrags][kWave], int st) {
     const int stage = st < all_stages ? st : 0;  // past the end: any stage, never multiplied
 #pragma unroll
     for (int i = 0; i < kAPer; ++i) {
-      const int col = (stage * KS + (wave + kWaves * i) % KS) * 32;  // + (lane / 16) * 8 in asrc
-      SHK_LOAD_TO_LDS(asrc[i] + (col + (lane / 16) * 8 < k ? col : 0), &buf[kWFrags + wave + kWaves * i][0]);
+      // (+ the lane's chunk, which is in asrc)
+      const int col = kUnits ? stage * 64 : (stage * KS + (wave + kWaves * i) % KS) * 32;
+      SHK_LOAD_TO_LDS(asrc[i] + (col + (kUnits ? lane / 8 : lane / 16) * 8 < k ? col : 0),
+                      &buf[kWFrags + wave + kWaves * i][0]);
     }
 #pragma unroll
     for (int i = 0; i < kWPer; ++i) {
@@ -785,7 +796,9 @@ __global__ void __launch_bounds__(GM* GN* kWave) __attribute__((amdgpu_waves_per
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-      for (int jn = 0; jn < WN; ++jn) af[ks][jn] = buf[kWFrags + (wn * WN + jn) * KS + ks][lane];
+      for (int jn = 0; jn < WN; ++jn)
+        af[ks][jn] = kUnits ? buf[kWFrags + (wn * WN + jn) * 2 + xunit][xplace + 32 * ks]
+                            : buf[kWFrags + (wn * WN + jn) * KS + ks][lane];
 #pragma unroll
       for (int i = 0; i < WM; ++i) wf[ks][i] = buf[(wm * WM + i) * KS + ks][lane];
     }

@@ -436,7 +436,11 @@ def test_gemm_tiled_weight(ops, n, m, k):
     [(1000, 16384, 288, False),  # tiles of 256 x 256, the last token tile partly empty
      (2048, 3584, 192, False),   # tiles of 256 x 128, stages of 64: three of them
      (2000, 3600, 448, False),   # the same with a partly empty tile on both sides, seven stages
-     (1000, 8192, 352, True)],   # gated, 256 x 256, eleven stages
+     (1000, 8192, 352, True),    # gated, 256 x 256, eleven stages
+     # stages of 64 whose activations arrive as units of 8 tokens x 128 bytes: the last unit of
+     # tokens partly empty, the last tile of k partly beyond k (its lanes fetch column 0)
+     (1997, 3600, 424, False),
+     (500, 2048, 616, False)],   # tiles of 128 x 128, eight wavefronts
 )
 def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
     """The large tiles with aligned rows and whole stages of k: operands go from
@@ -461,9 +465,10 @@ def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
     ops.gemm_tiled_weight(dev(a, dtype), wt, m, k, out, bias=dev(b))
     close(out, want, dtype)
     # a row's result does not depend on the rows around it
+    first = min(500, n - 300)
     part = torch.empty(300, m, device="cuda", dtype=dtype)
-    ops.gemm_tiled_weight(dev(a, dtype)[500:800], wt, m, k, part, bias=dev(b))
-    assert torch.equal(part, out[500:800])
+    ops.gemm_tiled_weight(dev(a, dtype)[first : first + 300], wt, m, k, part, bias=dev(b))
+    assert torch.equal(part, out[first : first + 300])
 
 
 def test_gemm_tiled_weight_rows_do_not_depend_on_the_rest_of_the_batch(ops):
