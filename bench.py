@@ -172,8 +172,8 @@ def run_prefill(engine, cfg, seed: int, repeats: int = 3) -> dict:
 
 def measure_peaks(device="cuda:0") -> dict:
     """What this GPU reaches on the plainest work of each kind: bytes per second
-    of a device-to-device copy of 2 GiB (read + write), of a read-only pass (a
-    sum) over the same buffer, and flop/s of the engine's own bfloat16 product
+    of a device-to-device copy of 2 GiB (read + write), of a read-only stream
+    (the engine's one-row product with a 1 GiB matrix), and flop/s of the engine's own bfloat16 product
     at 4096 x 4096 x 4096."""
     import torch
 
@@ -196,8 +196,14 @@ def measure_peaks(device="cuda:0") -> dict:
 
     nbytes = src.numel() * 2
     out["copy_gbs"] = round(2 * nbytes / timed(lambda: dst.copy_(src), 5) / 1e9, 1)
-    out["read_gbs"] = round(nbytes / timed(lambda: src.view(torch.int16).max(), 5) / 1e9, 1)
     del src, dst
+    # a read-only stream: the engine's own product of one row with a 1 GiB matrix
+    rows, width = 131072, 4096
+    big = ops.retile_weight(torch.empty(rows, width, dtype=torch.bfloat16, device=device).normal_())
+    x = torch.randn(1, width, device=device).to(torch.bfloat16)
+    y = torch.empty(1, rows, dtype=torch.bfloat16, device=device)
+    out["read_gbs"] = round(rows * width * 2 / timed(lambda: ops.gemm_tiled_weight(x, big, rows, width, y), 5) / 1e9, 1)
+    del big
     n = 4096
     a = torch.randn(n, n, device=device).to(torch.bfloat16)
     wt = ops.retile_weight(torch.randn(n, n, device=device).to(torch.bfloat16))

@@ -694,8 +694,8 @@ __global__ void __launch_bounds__(kWave) __attribute__((amdgpu_waves_per_eu(2)))
 // us.  Unit u < tiles * group is tile u / group, head u % group of the key/value
 // head.  The products are formed transposed as in the decode kernel (S^T = K Q^T,
 // O^T += V^T P^T): a lane owns one query, and P needs no trip through LDS.
-// grid (workgroup tiles, kv_heads); wg_seq / wg_q0 as tile_seq / tile_q0 above,
-// in steps of 16 * tiles queries.
+// grid (entries of wg_seq / wg_q0 x kv_heads); wg_seq / wg_q0 as tile_seq / tile_q0
+// above, in steps of 16 * tiles queries, in any order.
 
 constexpr int kUnitsPerWave = 1;
 // wavefronts per workgroup: 16, or 8 where that many would make too few workgroups
@@ -723,9 +723,10 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
   const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave;
   const int j = lane % 16, g = lane / 16;
   const PageDiv pd{page_size, page_magic};
-  // workgroups are listed in token order; the last ones read the most keys, so they start first
-  const int wg = gridDim.x - 1 - blockIdx.x;
-  const int seq = wg_seq[wg], q0 = wg_q0[wg], kvh = blockIdx.y;
+  // Workgroups start in the order of the host's list (every key/value head of an entry
+  // side by side): the host puts the entries that read the most keys first.
+  const int wg = blockIdx.x / kv_heads, kvh = blockIdx.x % kv_heads;
+  const int seq = wg_seq[wg], q0 = wg_q0[wg];
   const int group = heads / kv_heads;
   const int tok0 = cu_q[seq], q_len = cu_q[seq + 1] - tok0;
   const int start = ctx_lens[seq] - q_len;  // position of the portion's first token
@@ -1076,7 +1077,8 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
   const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim, small);
   SHK_REQUIRE(tiles > 0, "attention_prefill_shared: %d query heads per key/value head or head_dim %d "
               "is not served", heads / kv_heads, head_dim);
-  SHK_REQUIRE(num_wgs >= 0 && kv_heads <= 65535, "attention_prefill_shared: bad sizes");
+  SHK_REQUIRE(num_wgs >= 0 && static_cast<long long>(num_wgs) * kv_heads < (1ll << 31),
+              "attention_prefill_shared: bad sizes");
   if (num_wgs == 0) return 0;
   SHK_REQUIRE(q && out && cu_q && ctx_lens && wg_seq && wg_q0 && tables && k_pool && v_pool &&
                   table_stride > 0,
@@ -1087,7 +1089,7 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
               "attention_prefill_shared: a block table of %d pages of %d is beyond the kernel's range",
               table_stride, page_size);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(num_wgs, kv_heads);
+  dim3 grid(num_wgs * kv_heads);
 #define CALL(D)                                                                                \
   launch_prefill_shared<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
                            heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,      \

@@ -703,6 +703,9 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
         for q0 in range(0, l, 16 * tiles):
             wg_seq.append(s)
             wg_q0.append(q0)
+    # the kernel takes the list in any order (the engine sends the heaviest entries first)
+    mixed = torch.randperm(len(wg_seq), generator=torch.Generator().manual_seed(3)).tolist()
+    wg_seq, wg_q0 = [wg_seq[i] for i in mixed], [wg_q0[i] for i in mixed]
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
     out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
     scale = head_dim**-0.5

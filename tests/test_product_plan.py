@@ -96,3 +96,25 @@ def test_decode_graphs_are_keyed_by_buckets_and_few():
     assert runner._graph_key([StepEntry(seqs[0], [0], 0, [])]) is None
     assert runner._graph_key([StepEntry(seqs[0], [0], 0, [0])] * 257) is None
     assert np.all([len(v) >= 1 for v in keys.values()])
+
+
+def test_prompt_portions_are_launched_heaviest_first():
+    """The list of workgroups that the attention part hands to the prefill
+    kernel: runs of queries of every portion, each exactly once, the one whose
+    last query reads the most keys first."""
+    import numpy as np
+
+    from shrike_amd.parts.attention import QUERY_TILE, heavy_first, portion_runs
+
+    q_lens, starts = np.array([1, 1, 300, 40, 2048]), np.array([77, 5, 1900, 0, 0])
+    run = 2 * QUERY_TILE
+    seqs, q0 = portion_runs(q_lens[2:], 2, run)
+    assert sorted(zip(seqs.tolist(), q0.tolist())) == (
+        [(2, q) for q in range(0, 300, run)] + [(3, q) for q in range(0, 40, run)] + [(4, q) for q in range(0, 2048, run)])
+    keys = starts[seqs] + q0 + run
+    order = heavy_first(keys)
+    assert sorted(order.tolist()) == list(range(seqs.size))
+    assert (np.diff(keys[order]) <= 0).all()
+    # the 300-token portion at position 1,900 reads more keys than the whole prompt's last run
+    assert seqs[order][0] == 2 and q0[order][0] == 288
+    assert (seqs[order][-1], q0[order][-1]) in ((3, 0), (4, 0))
