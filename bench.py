@@ -204,6 +204,10 @@ def measure_peaks(device="cuda:0") -> dict:
     y = torch.empty(1, rows, dtype=torch.bfloat16, device=device)
     out["read_gbs"] = round(rows * width * 2 / timed(lambda: ops.gemm_tiled_weight(x, big, rows, width, y), 5) / 1e9, 1)
     del big
+    # the matrix units alone on random operands: the power limit's ceiling for every product
+    operands = torch.randn(32768, device=device).to(torch.bfloat16)
+    flop = ops.mfma_alone(operands, 2048, 2048)
+    out["mfma_tflops"] = round(flop / timed(lambda: ops.mfma_alone(operands, 2048, 2048), 3) / 1e12, 1)
     n = 4096
     a = torch.randn(n, n, device=device).to(torch.bfloat16)
     wt = ops.retile_weight(torch.randn(n, n, device=device).to(torch.bfloat16))
@@ -402,6 +406,7 @@ def main() -> int:
     if peaks:
         print(f"[bench] this GPU: {peaks}", file=sys.stderr)
         prefill["gemm_tflops"] = peaks["gemm_tflops"]
+        prefill["mfma_tflops"] = peaks["mfma_tflops"]  # the matrix units alone, random operands
         prefill["achievable_frac"] = round(
             prefill_flops(cfg, PROMPT_LEN) / (prefill["ms"] * 1e-3) / (peaks["gemm_tflops"] * 1e12), 4)
 

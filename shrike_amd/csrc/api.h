@@ -63,6 +63,12 @@ int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const float* bias,
                                int gated, int ksplit, void* stream);
 int shk_gemm_bf16_splits(int n, int m, int k);
 
+// The matrix instruction alone, for measuring its rate on operands of a given kind:
+// workgroups x 4 wavefronts each multiply, iters times, a 64 x 64 x 32 block
+// (2 * 64 * 64 * 32 flop) from `operands` (64 KiB of bfloat16), kept in registers.
+// out: workgroups * 256 floats.
+int shk_mfma_alone(const void* operands, float* out, int workgroups, int iters, void* stream);
+
 // Position encoding and cache write for the n tokens of a step.  qkv is
 // [n, (heads + 2*kv_heads) * head_dim]: queries, keys, values.  Queries and
 // keys are rotated by position (pairs (i, i + rot_dim/2), angle position *

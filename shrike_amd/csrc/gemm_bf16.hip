@@ -1072,6 +1072,41 @@ __global__ void __launch_bounds__(16 * kWave)
   }
 }
 
+// mfma_alone_kernel: the matrix instruction by itself, a 64 x 64 x 32 block per
+// wavefront and iteration from operands that stay in registers.  What it reaches is
+// the ceiling of every product kernel on this chip: with random operands the power
+// limit holds the clock well below the one that the published peak assumes, with
+// zeros it does not.
+__global__ void __launch_bounds__(4 * kWave)
+    mfma_alone_kernel(const u32x4* __restrict__ operands, float* __restrict__ out, int iters) {
+  const int tid = threadIdx.x;
+  u32x4 a[4], b[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    a[i] = operands[(tid + 64 * i) % 4096];
+    b[i] = operands[(tid * 3 + 64 * i + 7) % 4096];
+  }
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a[i]),
+                                                             __builtin_bit_cast(bf16x8, b[j]), acc[i][j], 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) sum += acc[i][j][0] + acc[i][j][3];
+  out[blockIdx.x * blockDim.x + tid] = sum;
+}
+
 }  // namespace shk
 
 using namespace shk;
@@ -1421,5 +1456,18 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
 #undef SHK_SKINNY
 #undef SHK_SKINNY_W
   SHK_LAUNCH_CHECK("gemm_bf16");
+  return 0;
+}
+
+// The matrix units alone: workgroups x 4 wavefronts, each iters times a 64 x 64 x 32
+// block (2 * 64 * 64 * 32 flop) from operands (64 KiB of bfloat16) held in registers;
+// out takes workgroups * 256 floats.  For measuring what the chip's matrix units give
+// on operands of a given kind; no product of the engine calls it.
+extern "C" int shk_mfma_alone(const void* operands, float* out, int workgroups, int iters, void* stream) {
+  SHK_REQUIRE(operands && out && workgroups > 0 && iters > 0, "mfma_alone: bad arguments");
+  SHK_REQUIRE(reinterpret_cast<uintptr_t>(operands) % 16 == 0, "mfma_alone: operands are not 16-byte aligned");
+  mfma_alone_kernel<<<workgroups, 4 * kWave, 0, static_cast<hipStream_t>(stream)>>>(
+      static_cast<const u32x4*>(operands), out, iters);
+  SHK_LAUNCH_CHECK("mfma_alone");
   return 0;
 }

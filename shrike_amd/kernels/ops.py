@@ -171,6 +171,18 @@ def gemm_splits(n: int, m: int, k: int) -> int:
     return int(load().shk_gemm_bf16_splits(n, m, k))
 
 
+def mfma_alone(operands: torch.Tensor, workgroups: int, iters: int) -> float:
+    """Runs the bfloat16 matrix instruction by itself on `operands` (at least
+    32,768 bfloat16 values, held in registers) and returns the flop it did:
+    for measuring what the matrix units give on operands of a given kind."""
+    if operands.dtype != torch.bfloat16 or operands.numel() < 32768 or not operands.is_contiguous():
+        raise KernelError("mfma_alone: operands must be 32,768 contiguous bfloat16 values or more")
+    out = torch.empty(workgroups * 256, dtype=torch.float32, device=operands.device)
+    check(load().shk_mfma_alone(_dev(operands, "operands"), _dev(out, "out", torch.float32), workgroups, iters,
+                                _stream()))
+    return 2.0 * 64 * 64 * 32 * 4 * workgroups * iters
+
+
 def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, gated=False,
                       splits: int = 1) -> None:
     """out (+)= a @ w.T + bias with wt = retile_weight(w): up to 64 rows of a

@@ -471,6 +471,18 @@ def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
     assert torch.equal(part, out[first : first + 300])
 
 
+def test_matrix_units_alone(ops):
+    """The measuring kernel behind the benchmark's `mfma_tflops`: it runs, says how
+    many flop it did, and refuses operands that would be read out of bounds."""
+    from shrike_amd.kernels.ops import KernelError
+
+    operands = torch.randn(32768, device="cuda").to(torch.bfloat16)
+    assert ops.mfma_alone(operands, 4, 3) == 2.0 * 64 * 64 * 32 * 4 * 4 * 3
+    torch.cuda.synchronize()
+    with pytest.raises(KernelError):
+        ops.mfma_alone(operands[:1000], 1, 1)
+
+
 def test_gemm_tiled_weight_rows_do_not_depend_on_the_rest_of_the_batch(ops):
     """Within one kernel (up to 16 rows, 17 to 64, more) a row's result is bit
     for bit the same whatever else is in the call; between kernels the order of
