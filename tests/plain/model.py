@@ -114,9 +114,10 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = No
 
 
 def causal_attention(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, window: int | None = None, first: int = 0
 ) -> torch.Tensor:
-    """q: [N, H, D]; k, v: [N, Hkv, D] of one whole sequence -> [N, H, D].
+    """q: [N - first, H, D], the queries at positions first .. N-1; k, v:
+    [N, Hkv, D] of one whole sequence -> [N - first, H, D].
 
     Query head h reads KV head h // (H // Hkv) (model_runner.py:129,
     triton_attention.py:43); scores are (q.k) * D**-0.5 (model_runner.py:131);
@@ -124,13 +125,14 @@ def causal_attention(
     kept keys; output sum_j a_j v_j.  With `window` a query also needs
     p - j < window (not in the reference).
     """
-    n, h, d = q.shape
+    n, (m, h, d) = k.shape[0], q.shape
+    assert m == n - first
     groups = h // k.shape[1]
     out = torch.empty_like(q)
-    pos = torch.arange(n)
-    keep = pos[None, :] <= pos[:, None]
+    pos_q, pos_k = torch.arange(first, n), torch.arange(n)
+    keep = pos_k[None, :] <= pos_q[:, None]
     if window is not None:
-        keep &= (pos[:, None] - pos[None, :]) < window
+        keep &= (pos_q[:, None] - pos_k[None, :]) < window
     for head in range(h):
         kv = head // groups
         scores = (q[:, head, :] @ k[:, kv, :].t()) * d**-0.5

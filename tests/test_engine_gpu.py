@@ -181,6 +181,45 @@ def test_long_decoding_and_first_tokens(model_root):
         cache.check([])
 
 
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol):
+    """A 10,000-token prompt in portions of up to 4,096 tokens (the later ones
+    read keys far back, through block tables of more than 600 pages), then six
+    single tokens from a graph with the key splits the engine chooses there."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    model_dir = make_model_dir("B", model_root, dtype=dtype, mode="unit")
+    ids = prompts_for("B", [10006], seed=9)[0]
+    wanted = {0: [0, 4095], 4096: [0, 4095], 8192: [0, 1807]}  # portion start -> rows within it
+    rows = [start + r for start, rs in wanted.items() for r in rs] + list(range(10000, 10006))
+    want = PlainModel(model_dir).logits(ids, rows=rows).double()
+    model, rt, _ = load_model(model_dir, dtype)
+    cache = CacheManager(model.cache_specs(), 16, 640, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    for g in cache.groups:  # a slot that is read before it is written shows up as NaN
+        g.k_tensor.fill_(float("nan"))
+        g.v_tensor.fill_(float("nan"))
+    runner = ModelRunner(model, cache, rt)
+    seq = cache.new_sequence()
+    got = []
+    for start, rs in wanted.items():
+        n = min(4096, 10000 - start)
+        cache.append(seq, start, n)
+        got.append(runner.step([StepEntry(seq, ids[start : start + n], start, rs)]).cpu().double())
+    for p in range(10000, 10006):
+        cache.append(seq, p, 1)
+        got.append(runner.step([StepEntry(seq, [ids[p]], p, [0])]).cpu().double())
+    assert runner.graph_replays == 6
+    got = torch.cat(got)
+    assert torch.isfinite(got).all()
+    err = (got - want).abs().amax(-1) / want.abs().max()
+    assert float(err.max()) <= tol, f"worst at row {rows[int(err.argmax())]}: {float(err.max()):.3e}"
+    cache.free(seq)
+    cache.check([])
+
+
 def test_add_request_guards(model_root):
     # tests/test_review_regressions.py:90-93
     from shrike_amd import SamplingParams

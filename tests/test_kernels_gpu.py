@@ -199,13 +199,11 @@ def reference_attention(q, k_pool, v_pool, tables, seq_lens, starts, page_size, 
         ctx = start + n_new
         pages = tables[s, : -(-ctx // page_size)].long().cpu()
         # [pages, kv_heads, slabs, page_size, slab] -> [keys, kv_heads, head_dim]
-        k = k_pool.cpu().double()[pages].permute(0, 3, 1, 2, 4).reshape(-1, k_pool.shape[1], k_pool.shape[2] * k_pool.shape[4])[:ctx]
-        v = v_pool.cpu().double()[pages].permute(0, 3, 1, 2).reshape(-1, v_pool.shape[1], v_pool.shape[2])[:ctx]
+        k = k_pool[pages.to(k_pool.device)].cpu().double().permute(0, 3, 1, 2, 4).reshape(-1, k_pool.shape[1], k_pool.shape[2] * k_pool.shape[4])[:ctx]
+        v = v_pool[pages.to(v_pool.device)].cpu().double().permute(0, 3, 1, 2).reshape(-1, v_pool.shape[1], v_pool.shape[2])[:ctx]
         k, v = torch.nan_to_num(k), torch.nan_to_num(v)  # slots outside the window may be poisoned
-        full_q = torch.zeros(ctx, heads, q.shape[2], dtype=torch.float64)
-        full_q[start:] = q[off : off + n_new]
         d = q.shape[2]
-        o = plain.causal_attention(full_q * (scale / d**-0.5), k, v, window)[start:]
+        o = plain.causal_attention(q[off : off + n_new].double() * (scale / d**-0.5), k, v, window, first=start)
         outs.append(o)
         off += n_new
     return torch.cat(outs)
@@ -802,17 +800,70 @@ def test_attention_prefill_over_two_thousand_keys(ops, heads, kv_heads, kernel):
         assert (got[row, head].double().cpu() - v).abs().max() <= 2e-2 * v.abs().max(), (s, p, j)
 
 
-def test_attention_decode_finds_far_keys_in_a_long_context(ops):
-    """Single tokens at contexts up to 4,100 with the key splits the engine would
-    choose for them; every sequence has one key whose score stands out, at the
-    start, at a split's edge, at the very end."""
+@pytest.mark.parametrize("kernel", ["shared", "tiles"])
+def test_attention_prefill_of_portions_far_into_a_sequence(ops, kernel):
+    """Prompt portions that start at positions 30,000 and 16,000 (a long prompt cut
+    by the token budget): their queries read thousands of keys written by earlier
+    steps; chosen queries have one key that stands out, at the sequence's start, at
+    the portion's own start, just before it."""
+    torch.manual_seed(33)
+    dtype = torch.bfloat16
+    heads, kv_heads, head_dim, page_size, group = 28, 4, 128, 16, 7
+    seq_lens, starts = [200, 64], [30000, 16000]
+    ctx = [s + l for s, l in zip(starts, seq_lens)]
+    n = sum(seq_lens)
+    tables, k_pool, v_pool = paged_setup(ctx, page_size, sum(-(-c // page_size) for c in ctx) + 3, kv_heads,
+                                         head_dim, dtype, seed=8)
+    q = torch.randn(n, heads, head_dim) * 0.3
+    keys = [torch.randn(c, kv_heads, head_dim) * 0.3 for c in ctx]
+    values = [torch.randn(c, kv_heads, head_dim) for c in ctx]
+    pairs = [(0, 30000, 0), (0, 30199, 29999), (0, 30100, 30000), (0, 30017, 15000), (0, 30150, 30150),
+             (1, 16000, 15999), (1, 16063, 31), (1, 16032, 16000)]
+    for i, (s, p, j) in enumerate(pairs):
+        u = torch.zeros(head_dim)
+        u[(7 * i) % head_dim] = 20.0
+        head = (3 * i) % heads
+        q[sum(seq_lens[:s]) + p - starts[s], head] = u
+        keys[s][j, head // group] = u
+    for s in range(2):
+        fill_pools_from(tables, k_pool, v_pool, s, keys[s], values[s], page_size)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
+    out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
+    scale = head_dim**-0.5
+    run = 16 * (ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim, small=True) if kernel == "shared" else 1)
+    wg_seq = [s for s, l in enumerate(seq_lens) for _ in range(0, l, run)]
+    wg_q0 = [q0 for l in seq_lens for q0 in range(0, l, run)]
+    args = (i32([0, 200, n]), i32(ctx), i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, None, scale)
+    qd = dev(q.to(dtype)).view(n, -1)
+    if kernel == "shared":
+        ops.attention_prefill_shared(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args, small=True)
+    else:
+        ops.attention_prefill(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args)
+    want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, seq_lens, starts, page_size, None, scale)
+    assert not torch.isnan(out.float()).any()
+    got = out.view(n, heads, head_dim)
+    close(got, want, dtype, scale=1.0)
+    for i, (s, p, j) in enumerate(pairs):
+        row, head = sum(seq_lens[:s]) + p - starts[s], (3 * i) % heads
+        v = values[s][j, head // group].to(dtype).double()
+        assert (got[row, head].double().cpu() - v).abs().max() <= 2e-2 * v.abs().max(), (s, p, j)
+
+
+@pytest.mark.parametrize(
+    "ctx, special",
+    [([4100, 4096, 2049, 2048, 1025, 300, 4097, 1], [0, 4095, 1023, 2047, 512, 299, 2048, 0]),
+     # block tables of 2,500 pages, the most key splits the kernel has
+     ([40000, 33001, 16385, 70], [0, 33000, 8192, 69])],
+)
+def test_attention_decode_finds_far_keys_in_a_long_context(ops, ctx, special):
+    """Single tokens at contexts up to 4,100 and up to 40,000 with the key splits
+    the engine would choose for them; every sequence has one key whose score
+    stands out, at the start, at a split's edge, at the very end."""
     from shrike_amd.parts.attention import decode_splits
 
     torch.manual_seed(32)
     dtype = torch.bfloat16
     heads, kv_heads, head_dim, page_size, group = 28, 4, 128, 16, 7
-    ctx = [4100, 4096, 2049, 2048, 1025, 300, 4097, 1]
-    special = [0, 4095, 1023, 2047, 512, 299, 2048, 0]
     n = len(ctx)
     tables, k_pool, v_pool = paged_setup(ctx, page_size, sum(-(-c // page_size) for c in ctx) + 3, kv_heads,
                                          head_dim, dtype, seed=7)

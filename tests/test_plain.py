@@ -143,3 +143,14 @@ def test_sampler_vectors_of_the_reference():
     # mass before an entry below top_p: [0.5, 0.3, 0.2], top_p 0.6 keeps two
     ids, _ = plain.softmax_sample_reference(torch.log(torch.tensor([0.2, 0.5, 0.3])), 1.0, 0.6)
     assert ids.tolist() == [1, 2]
+
+
+def test_attention_of_the_last_queries_alone():
+    """`first`: only the queries from that position on, against the rows of the whole."""
+    torch.manual_seed(5)
+    n, h, hkv, d = 23, 6, 2, 8
+    q, k, v = torch.randn(n, h, d).double(), torch.randn(n, hkv, d).double(), torch.randn(n, hkv, d).double()
+    for window in (None, 5):
+        whole = plain.causal_attention(q, k, v, window)
+        for first in (0, 1, 17, 22):
+            assert torch.allclose(plain.causal_attention(q[first:], k, v, window, first=first), whole[first:], atol=1e-13)
