@@ -130,6 +130,12 @@ int shk_attention_prefill_bf16(const void* q, int q_stride, void* out, int num_t
 // half as many tiles each, for portions that would otherwise make too few
 // workgroups for the chip.  tiles == 0: the shape is not served (more query
 // heads per key/value head than a workgroup has wavefronts, head_dim > 128).
+// Entries are launched in the order of the list.  nsplit > 1 shares every entry's
+// keys among nsplit workgroups (for a few queries far into a sequence, which alone
+// would leave most of the chip idle); their results go through `partial`
+// (prompt_tokens * heads * nsplit * (head_dim + 2) floats) and are merged into out.
+// first_token: the index of the step's first prompt token (prompt tokens follow
+// the single tokens); prompt_tokens: how many there are.
 int shk_attention_prefill_shared_tiles(int heads, int kv_heads, int head_dim, int small);
 int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out, int num_wgs,
                                       int heads, int kv_heads, int head_dim, const int32_t* cu_q,
@@ -137,7 +143,8 @@ int shk_attention_prefill_shared_bf16(const void* q, int q_stride, void* out, in
                                       const int32_t* wg_q0, const int32_t* tables,
                                       int table_stride, const void* k_pool, const void* v_pool,
                                       int page_size, int window, float scale, int small,
-                                      void* stream);
+                                      float* partial, int nsplit, int first_token,
+                                      int prompt_tokens, void* stream);
 
 // out[r] = lowest index of the largest value of logits[r, :vocab].  Rows wider
 // than 4096 are searched in chunks; scratch then holds

@@ -712,7 +712,9 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
                                     const int32_t* __restrict__ wg_q0,
                                     const int32_t* __restrict__ tables, int table_stride,
                                     const bf16* __restrict__ k_pool, const bf16* __restrict__ v_pool,
-                                    int page_size, uint32_t page_magic, int window, float scale) {
+                                    int page_size, uint32_t page_magic, int window, float scale,
+                                    float* __restrict__ partial, int nsplit, int first_token,
+                                    int partial_rows) {
   constexpr int U = kUnitsPerWave;
   constexpr int kKFrags = 2 * (D / 32), kVFrags = D / 16, kFrags = kKFrags + kVFrags;
   // fragments each wavefront stages; where they do not divide, some are staged twice
@@ -725,7 +727,8 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
   const PageDiv pd{page_size, page_magic};
   // Workgroups start in the order of the host's list (every key/value head of an entry
   // side by side): the host puts the entries that read the most keys first.
-  const int wg = blockIdx.x / kv_heads, kvh = blockIdx.x % kv_heads;
+  const int z = blockIdx.x % nsplit;  // which share of the entry's keys
+  const int wg = blockIdx.x / (nsplit * kv_heads), kvh = (blockIdx.x / nsplit) % kv_heads;
   const int seq = wg_seq[wg], q0 = wg_q0[wg];
   const int group = heads / kv_heads;
   const int tok0 = cu_q[seq], q_len = cu_q[seq + 1] - tok0;
@@ -739,6 +742,11 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
   const int lo_min = (window > 0 && pos_min - window + 1 > 0) ? pos_min - window + 1 : 0;
   const int key_begin = lo_min & ~31;
   const int nchunks = (pos_max - key_begin) / 32 + 1;
+  // this workgroup's share of the chunks (all of them without splits; none at all
+  // for the last shares of an entry with few keys)
+  const int per_split = (nchunks + nsplit - 1) / nsplit;
+  const int c_first = z * per_split;
+  const int c_end = c_first + per_split < nchunks ? c_first + per_split : nchunks;
 
   // this wavefront's units; a lane owns query j of each
   AFrag qf[U][D / 32];
@@ -900,27 +908,29 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
   // Chunk c is multiplied from LDS buffer c % 2 while the loads of chunks c + 1 and
   // c + 2 are in flight.  The loop's body has no branch, so the loads stay where
   // they are written.
-  u32x4 even[kPer], odd[kPer];
-  fetch(even, 0);
-  fetch(odd, 1);
-  put(even, 0, 0);
-  __syncthreads();
-  int c = 0;
-  for (; c + 2 < nchunks; c += 2) {
-    fetch(even, c + 2);
+  if (c_first < c_end) {  // the same for every wavefront of the workgroup
+    u32x4 even[kPer], odd[kPer];
+    fetch(even, c_first);
+    fetch(odd, c_first + 1);
+    put(even, c_first, 0);
+    __syncthreads();
+    int c = c_first;
+    for (; c + 2 < c_end; c += 2) {
+      fetch(even, c + 2);
+      attend(0, c);
+      put(odd, c + 1, 1);
+      __syncthreads();
+      fetch(odd, c + 3);
+      attend(1, c + 1);
+      put(even, c + 2, 0);
+      __syncthreads();
+    }
     attend(0, c);
-    put(odd, c + 1, 1);
-    __syncthreads();
-    fetch(odd, c + 3);
-    attend(1, c + 1);
-    put(even, c + 2, 0);
-    __syncthreads();
-  }
-  attend(0, c);
-  if (c + 1 < nchunks) {
-    put(odd, c + 1, 1);
-    __syncthreads();
-    attend(1, c + 1);
+    if (c + 1 < c_end) {
+      put(odd, c + 1, 1);
+      __syncthreads();
+      attend(1, c + 1);
+    }
   }
 
 #pragma unroll
@@ -929,6 +939,20 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
     total += __shfl_xor(total, 16, kWave);
     total += __shfl_xor(total, 32, kWave);
     if (j >= unit_rows[u]) continue;
+    if (nsplit > 1) {
+      // a share's result, for attention_merge_kernel: O [row][share][D], then (maximum,
+      // sum) [row][share][2], row = the token's index among the step's prompt tokens x head
+      const size_t row = static_cast<size_t>(tok0 + unit_q0[u] + j - first_token) * heads + unit_head[u];
+      float* dst = partial + (row * nsplit + z) * D + 4 * g;
+#pragma unroll
+      for (int db = 0; db < D / 16; ++db)
+        *reinterpret_cast<float4*>(dst + db * 16) =
+            make_float4(o[u][db][0], o[u][db][1], o[u][db][2], o[u][db][3]);
+      if (g == 0)
+        *reinterpret_cast<float2*>(partial + static_cast<size_t>(partial_rows) * nsplit * D +
+                                   (row * nsplit + z) * 2) = make_float2(m[u], total);
+      continue;
+    }
     const float inv = 1.f / total;
     bf16* dst = out + static_cast<size_t>(tok0 + unit_q0[u] + j) * heads * D +
                 static_cast<size_t>(unit_head[u]) * D + 4 * g;
@@ -975,16 +999,23 @@ static void launch_prefill_shared(dim3 grid, hipStream_t s, const bf16* q, int q
                                   const int32_t* ctx_lens, const int32_t* wg_seq,
                                   const int32_t* wg_q0, const int32_t* tables, int table_stride,
                                   const bf16* k_pool, const bf16* v_pool, int page_size, int window,
-                                  float scale, bool small) {
+                                  float scale, bool small, float* partial, int nsplit,
+                                  int first_token, int prompt_tokens) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
+  const int rows = prompt_tokens * heads;
   if (small)
     attention_prefill_shared_kernel<D, kSharedWavesSmall><<<grid, kSharedWavesSmall * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
-        table_stride, k_pool, v_pool, page_size, magic, window, scale);
+        table_stride, k_pool, v_pool, page_size, magic, window, scale, partial, nsplit, first_token,
+        rows);
   else
     attention_prefill_shared_kernel<D, kSharedWaves><<<grid, kSharedWaves * kWave, 0, s>>>(
         q, q_stride, out, heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,
-        table_stride, k_pool, v_pool, page_size, magic, window, scale);
+        table_stride, k_pool, v_pool, page_size, magic, window, scale, partial, nsplit, first_token,
+        rows);
+  if (nsplit > 1)
+    attention_merge_kernel<D><<<rows, kWave, 0, s>>>(
+        partial, out + static_cast<size_t>(first_token) * heads * D, nsplit);
 }
 
 }  // namespace shk
@@ -1071,15 +1102,23 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
                                                  const int32_t* wg_q0, const int32_t* tables,
                                                  int table_stride, const void* k_pool,
                                                  const void* v_pool, int page_size, int window,
-                                                 float scale, int small, void* stream) {
+                                                 float scale, int small, float* partial, int nsplit,
+                                                 int first_token, int prompt_tokens, void* stream) {
   if (check_mfma_shapes("attention_prefill_shared", heads, kv_heads, head_dim, page_size, q_stride))
     return 1;
   const int tiles = shk_attention_prefill_shared_tiles(heads, kv_heads, head_dim, small);
   SHK_REQUIRE(tiles > 0, "attention_prefill_shared: %d query heads per key/value head or head_dim %d "
               "is not served", heads / kv_heads, head_dim);
-  SHK_REQUIRE(num_wgs >= 0 && static_cast<long long>(num_wgs) * kv_heads < (1ll << 31),
+  SHK_REQUIRE(nsplit >= 1 && nsplit <= kMaxSplits, "attention_prefill_shared: %d key splits (at most %d)",
+              nsplit, kMaxSplits);
+  SHK_REQUIRE(num_wgs >= 0 && static_cast<long long>(num_wgs) * kv_heads * nsplit < (1ll << 31),
               "attention_prefill_shared: bad sizes");
   if (num_wgs == 0) return 0;
+  SHK_REQUIRE(nsplit == 1 || (partial && first_token >= 0 && prompt_tokens > 0 &&
+                              reinterpret_cast<uintptr_t>(partial) % 16 == 0 &&
+                              static_cast<long long>(prompt_tokens) * heads < (1ll << 31)),
+              "attention_prefill_shared: key splits need a 16-byte aligned partial buffer, the index "
+              "of the first prompt token and the number of prompt tokens");
   SHK_REQUIRE(q && out && cu_q && ctx_lens && wg_seq && wg_q0 && tables && k_pool && v_pool &&
                   table_stride > 0,
               "attention_prefill_shared: null pointer");
@@ -1089,12 +1128,13 @@ extern "C" int shk_attention_prefill_shared_bf16(const void* q, int q_stride, vo
               "attention_prefill_shared: a block table of %d pages of %d is beyond the kernel's range",
               table_stride, page_size);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  dim3 grid(num_wgs * kv_heads);
+  dim3 grid(num_wgs * kv_heads * nsplit);
 #define CALL(D)                                                                                \
   launch_prefill_shared<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), \
                            heads, kv_heads, tiles, cu_q, ctx_lens, wg_seq, wg_q0, tables,      \
                            table_stride, static_cast<const bf16*>(k_pool),                     \
-                           static_cast<const bf16*>(v_pool), page_size, window, scale, small != 0)
+                           static_cast<const bf16*>(v_pool), page_size, window, scale, small != 0, \
+                           partial, nsplit, first_token, prompt_tokens)
   switch (head_dim) {
     case 32: CALL(32); break;
     case 64: CALL(64); break;

@@ -32,7 +32,8 @@ _SIGNATURES = {
     "shk_attention_decode_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _I, _F, _P, _I, _P],
     "shk_attention_prefill_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _P],
     "shk_attention_prefill_shared_tiles": [_I, _I, _I, _I],
-    "shk_attention_prefill_shared_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _P],
+    "shk_attention_prefill_shared_bf16": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _I,
+                                          _P, _I, _I, _I, _P],
     "shk_argmax": [_P, _P, _I, _I, _I, _P, _P],
     "shk_argmax_scratch_floats": [_I, _I],
     "shk_sample": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],

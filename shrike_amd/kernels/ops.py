@@ -357,10 +357,14 @@ def attention_prefill_shared_tiles(heads, kv_heads, head_dim, small=False) -> in
 
 
 def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, ctx_lens, wg_seq, wg_q0,
-                             tables, k_pool, v_pool, page_size, window, scale, small=False) -> None:
+                             tables, k_pool, v_pool, page_size, window, scale, small=False,
+                             partial=None, nsplit: int = 1, first_token: int = 0) -> None:
     """bfloat16 MFMA attention for prompt portions; one workgroup per (run of query
     tiles, key/value head) shares each chunk of keys among its query heads.
-    wg_seq / wg_q0 are in steps of 16 * attention_prefill_shared_tiles(..., small)."""
+    wg_seq / wg_q0 are in steps of 16 * attention_prefill_shared_tiles(..., small),
+    launched in the list's order.  nsplit > 1 shares every entry's keys among
+    that many workgroups, whose results pass through `partial` (float32, (rows
+    of q from first_token on) * heads * nsplit * (head_dim + 2) values)."""
     _rows(q, "attention_prefill_shared q")
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise KernelError("attention_prefill_shared: bfloat16 only")
@@ -369,13 +373,21 @@ def attention_prefill_shared(q, out, num_wgs, heads, kv_heads, head_dim, cu_q, c
     if wg_seq.shape[0] < num_wgs or wg_q0.shape[0] < num_wgs:
         raise KernelError("attention_prefill_shared: workgroup arrays are shorter than num_wgs")
     _check_pools("attention_prefill_shared", q, tables, k_pool, v_pool, kv_heads, head_dim, page_size)
+    prompt_tokens = q.shape[0] - first_token
+    if nsplit > 1:
+        need = prompt_tokens * heads * nsplit * (head_dim + 2)
+        if partial is None or partial.dtype != torch.float32 or partial.numel() < need or prompt_tokens <= 0:
+            raise KernelError(f"attention_prefill_shared: {nsplit} key splits need a float32 partial buffer "
+                              f"of {need} values for the {prompt_tokens} prompt tokens")
     check(
         load().shk_attention_prefill_shared_bf16(
             _dev(q, "q"), q.stride(0), _dev(out, "out"), num_wgs, heads, kv_heads, head_dim,
             _dev(cu_q, "cu_q", torch.int32), _dev(ctx_lens, "ctx_lens", torch.int32),
             _dev(wg_seq, "wg_seq", torch.int32), _dev(wg_q0, "wg_q0", torch.int32),
             _dev(tables, "tables", torch.int32), tables.shape[1], _dev(k_pool, "k_pool"),
-            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), int(small), _stream(),
+            _dev(v_pool, "v_pool"), page_size, int(window or 0), float(scale), int(small),
+            _dev(partial, "partial", torch.float32) if nsplit > 1 else None, int(nsplit), int(first_token),
+            int(prompt_tokens), _stream(),
         )
     )
 

@@ -45,6 +45,8 @@ class AttentionPlan:
     nsplit: int = 1  # key splits of the single-token rows
     kernel: str = ""  # for prompt portions: "shared", "tiles" or "" (none in the step)
     small: bool = False  # "shared" with half as many wavefronts per workgroup
+    portion_splits: int = 1  # "shared": workgroups that share an entry's keys
+    first_token: int = 0  # index of the step's first prompt token
     count: int = 0  # workgroups ("shared") or tiles ("tiles")
     seq_name: str = ""  # names of the launch lists among the step's extras
     q0_name: str = ""
@@ -59,6 +61,20 @@ def portion_runs(q_lens, first_seq: int, run: int):
     np.cumsum(counts, out=first[1:])
     q0 = (np.arange(int(counts.sum())) - first[seqs - first_seq]) * run
     return seqs, q0
+
+
+def portion_splits(workgroups: int, mean_keys: int) -> int:
+    """Among how many workgroups each entry of a step's prompt portions shares
+    its keys.  A few hundred queries far into a sequence (a long prompt cut by
+    the token budget) make few workgroups with thousands of keys each; shared,
+    they fill the chip.  Measured at 28 heads over 4, 512 queries (128
+    workgroups): at position 1,536 64 us a layer unshared, 47 / 40 / 48 in 2 / 4
+    / 8 shares; at 31,000 900 us against 464 / 337 / 345; from position 0 (264
+    keys on average) 21 us against 25 in 2.  Hence as many shares as bring the
+    launch to twice the compute units, each worth 256 keys or more on average."""
+    if workgroups <= 0:
+        return 1
+    return max(1, min(SMALL_WORKGROUPS_AT_ONCE // workgroups, mean_keys // KEYS_PER_WORKGROUP, MAX_KEY_SPLITS))
 
 
 def heavy_first(work):
@@ -182,8 +198,13 @@ class PagedAttention(Mixer):
                     plan.small, tiles = True, small_tiles
             seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE * tiles)
             # the keys an entry's last query reads: where its portion starts plus its queries
-            order = heavy_first(shape.starts[seqs] + q0 + QUERY_TILE * tiles)
+            keys = shape.starts[seqs] + q0 + QUERY_TILE * tiles
+            if s.window:
+                keys = np.minimum(keys, s.window + QUERY_TILE * tiles)
+            order = heavy_first(keys)
             seqs, q0 = seqs[order], q0[order]
+            plan.portion_splits = portion_splits(int(seqs.size) * hkv, int(keys.mean()))
+            plan.first_token = shape.num_decode
         else:
             plan.kernel = "tiles"
             seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE)
@@ -212,10 +233,16 @@ class PagedAttention(Mixer):
                                  cache.k_pool, cache.v_pool, cache.page_size, s.window, s.scale,
                                  partial, plan.nsplit)
         if plan.kernel == "shared":
+            partial = None
+            if plan.portion_splits > 1:
+                prompt_tokens = ctx.num_tokens - plan.first_token
+                partial = ctx.buffer("attn_portion_partial",
+                                     (prompt_tokens * h * plan.portion_splits * (d + 2),), torch.float32)
             ops.attention_prefill_shared(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                          ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
                                          cache.k_pool, cache.v_pool, cache.page_size, s.window,
-                                         s.scale, small=plan.small)
+                                         s.scale, small=plan.small, partial=partial,
+                                         nsplit=plan.portion_splits, first_token=plan.first_token)
         elif plan.kernel == "tiles":
             ops.attention_prefill(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                   ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,

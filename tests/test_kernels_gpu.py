@@ -686,11 +686,13 @@ def test_rope_kv_store_adds_up_a_split_product(ops, n, splits):
      (16, 2, 64, 16, 100), (3, 1, 128, 48, None), (16, 1, 32, 16, None), (12, 1, 64, 32, 50),
      (40, 8, 128, 16, None)],
 )
-@pytest.mark.parametrize("small", [False, True])
-def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window, small):
+@pytest.mark.parametrize("small, nsplit", [(False, 1), (True, 1), (True, 3), (False, 8)])
+def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window, small, nsplit):
     """The prefill kernel that shares each chunk of keys among the query heads of a
     key/value head: 1 to 16 heads per group, portions of 2 to 200 tokens, in
-    workgroups of 16 wavefronts and of 8 (`small`)."""
+    workgroups of 16 wavefronts and of 8 (`small`), every entry's keys in one
+    workgroup or shared among 3 or 8 (more shares than some entries have chunks
+    of keys: the last ones find nothing to do)."""
     torch.manual_seed(20)
     dtype = torch.bfloat16
     tiles = ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim, small)
@@ -719,9 +721,10 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
     out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
     scale = head_dim**-0.5
+    partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
     ops.attention_prefill_shared(dev(q).view(n, -1), out, len(wg_seq), heads, kv_heads, head_dim, i32(cu), i32(ctx),
                                  i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, window, scale,
-                                 small=small)
+                                 small=small, partial=partial, nsplit=nsplit)
     want = reference_attention(q.double(), k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale)
     assert not torch.isnan(out.float()).any()
     close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
@@ -835,8 +838,14 @@ def test_attention_prefill_of_portions_far_into_a_sequence(ops, kernel):
     wg_q0 = [q0 for l in seq_lens for q0 in range(0, l, run)]
     args = (i32([0, 200, n]), i32(ctx), i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, None, scale)
     qd = dev(q.to(dtype)).view(n, -1)
-    if kernel == "shared":
-        ops.attention_prefill_shared(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args, small=True)
+    if kernel == "shared":  # as the engine launches such a step: every entry's keys shared among workgroups
+        from shrike_amd.parts.attention import portion_splits
+
+        nsplit = portion_splits(len(wg_seq) * kv_heads, 23000)
+        assert nsplit > 1
+        partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
+        ops.attention_prefill_shared(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args, small=True,
+                                     partial=partial, nsplit=nsplit)
     else:
         ops.attention_prefill(qd, out, len(wg_seq), heads, kv_heads, head_dim, *args)
     want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, seq_lens, starts, page_size, None, scale)

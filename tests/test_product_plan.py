@@ -118,3 +118,13 @@ def test_prompt_portions_are_launched_heaviest_first():
     # the 300-token portion at position 1,900 reads more keys than the whole prompt's last run
     assert seqs[order][0] == 2 and q0[order][0] == 288
     assert (seqs[order][-1], q0[order][-1]) in ((3, 0), (4, 0))
+
+
+def test_shares_of_a_portions_keys():
+    from shrike_amd.parts.attention import portion_splits
+
+    assert portion_splits(512, 1000) == 1  # a whole 2,048-token prompt: enough workgroups already
+    assert portion_splits(128, 264) == 1   # 512 queries from position 0: too few keys to share
+    assert portion_splits(128, 1800) == 4 and portion_splits(256, 3600) == 2
+    assert portion_splits(32, 8000) == 16 and portion_splits(4, 100000) == 64
+    assert portion_splits(0, 5) == 1
