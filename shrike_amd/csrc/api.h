@@ -62,6 +62,9 @@ int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const float* bias,
                                int m, int k, int lda, int ldo, int out_dtype, int accumulate,
                                int gated, int ksplit, void* stream);
 int shk_gemm_bf16_splits(int n, int m, int k);
+// 2 where a product of many tokens runs as two (the weight rows whose tiles make whole
+// rounds of the compute units, then the rest with tiles of its own), else 1.
+int shk_gemm_bf16_parts(int n, int m, int k, int gated);
 
 // The matrix instruction alone, for measuring its rate on operands of a given kind:
 // workgroups x 4 wavefronts each multiply, iters times, a 64 x 64 x 32 block

@@ -1266,6 +1266,34 @@ static int big_shape(int split, int n, int wblocks, int m, int k) {
   return best;
 }
 
+extern "C" int shk_gemm_bf16_splits(int n, int m, int k);
+
+// 256 x 256 tiles that do not make whole rounds of the 256 compute units (296 of them:
+// two rounds, the second nearly empty) are better run as two products: the row tiles
+// that make whole rounds, then the remaining rows with the tile shape that suits them.
+// Returns how many blocks of 16 weight rows the first product takes, or 0 where the
+// estimate does not expect a tenth less time than from `shape` alone.
+static int big_main_blocks(int shape, int n, int wblocks, int m, int k, int gated) {
+  const int tiles_x = (wblocks + 15) / 16, tiles_y = (n + 255) / 256;
+  const long long total = static_cast<long long>(tiles_x) * tiles_y;
+  const int main_x = static_cast<int>(total / 256 * 256 / tiles_y);
+  if (total <= 256 || main_x <= 0 || main_x >= tiles_x) return 0;
+  const int main_blocks = main_x * 16, rest_blocks = wblocks - main_blocks;
+  const int main_rows = main_blocks * 16 / (gated ? 2 : 1), rest_rows = m - main_rows;
+  const int rest_shape = big_shape(1, n, rest_blocks, rest_rows, k);
+  const double whole = big_estimate(shape, 1, n, wblocks, m, k);
+  const double parts = big_estimate(0, 1, n, main_blocks, main_rows, k) +
+                       big_estimate(rest_shape, 1, n, rest_blocks, rest_rows, k);
+  return parts < 0.9 * whole ? main_blocks : 0;
+}
+
+// Products that a call with these sizes is made of (1, or 2: see big_main_blocks).
+extern "C" int shk_gemm_bf16_parts(int n, int m, int k, int gated) {
+  if (n <= 64 || shk_gemm_bf16_splits(n, m, k) > 1) return 1;
+  const int wblocks = (gated ? 2 : 1) * ((m + 15) / 16);
+  return big_main_blocks(big_shape(1, n, wblocks, m, k), n, wblocks, m, k, gated) ? 2 : 1;
+}
+
 extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   const int mblocks = (m + 15) / 16, ktiles = (k + 31) / 32;
   if (n > 64) {
@@ -1327,6 +1355,33 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
     // Tile of the workgroup: 256 x 256, 256 x 128 or 128 x 128 (weight rows x
     // tokens), whichever big_estimate() expects to finish first.
     const int shape = big_shape(ksplit, n, wblocks, m, k);
+    int main_blocks = 0;
+    if (ksplit == 1) main_blocks = big_main_blocks(shape, n, wblocks, m, k, gated);
+    if (main_blocks) {
+      const int rest_blocks = wblocks - main_blocks;
+      const int main_rows = main_blocks * 16 / (gated ? 2 : 1), rest_rows = m - main_rows;
+      const int rest_shape = big_shape(1, n, rest_blocks, rest_rows, k);
+      launch_big<4, 4, 4, 4, 1>(s, ap, lda, n, k, wp, kt, main_rows, bias, out, ldo, of, accumulate,
+                                vec, gated, main_blocks, 1);
+      const uint4* rest_w = wp + static_cast<size_t>(main_blocks) * kt * kWave;
+      const float* rest_bias = bias ? bias + main_rows : nullptr;
+      void* rest_out = of ? static_cast<void*>(static_cast<float*>(out) + main_rows)
+                          : static_cast<void*>(static_cast<bf16*>(out) + main_rows);
+      if (rest_shape == 0)
+        launch_big<4, 4, 4, 4, 1>(s, ap, lda, n, k, rest_w, kt, rest_rows, rest_bias, rest_out, ldo,
+                                  of, accumulate, vec, gated, rest_blocks, 1);
+      else if (rest_shape == 1)
+        launch_big<4, 4, 4, 2, 2>(s, ap, lda, n, k, rest_w, kt, rest_rows, rest_bias, rest_out, ldo,
+                                  of, accumulate, vec, gated, rest_blocks, 1);
+      else if (static_cast<long long>((rest_blocks + 7) / 8) * ((n + 127) / 128) <= 256)
+        launch_big<4, 2, 2, 4, 2>(s, ap, lda, n, k, rest_w, kt, rest_rows, rest_bias, rest_out, ldo,
+                                  of, accumulate, vec, gated, rest_blocks, 1);
+      else
+        launch_big<2, 2, 4, 4, 2>(s, ap, lda, n, k, rest_w, kt, rest_rows, rest_bias, rest_out, ldo,
+                                  of, accumulate, vec, gated, rest_blocks, 1);
+      SHK_LAUNCH_CHECK("gemm_bf16");
+      return 0;
+    }
     if (shape == 0)
       launch_big<4, 4, 4, 4, 1>(s, ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, vec,
                                 gated, wblocks, ksplit);

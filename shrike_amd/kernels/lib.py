@@ -25,6 +25,7 @@ _SIGNATURES = {
     "shk_interleave_gate_up": [_P, _P, _I, _I, _P, _P],
     "shk_gemm_bf16_tiled_weight": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "shk_gemm_bf16_splits": [_I, _I, _I],
+    "shk_gemm_bf16_parts": [_I, _I, _I, _I],
     "shk_mfma_alone": [_P, _P, _I, _I, _P],
     "shk_rope_kv_store": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _P, _I, _P, _P],
     "shk_attention": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _P],

@@ -171,6 +171,12 @@ def gemm_splits(n: int, m: int, k: int) -> int:
     return int(load().shk_gemm_bf16_splits(n, m, k))
 
 
+def gemm_parts(n: int, m: int, k: int, gated: bool = False) -> int:
+    """Launches that an [n, k] x [m, k]^T product is made of (2: rows whose tiles
+    fill whole rounds of the compute units, then the rest)."""
+    return int(load().shk_gemm_bf16_parts(n, m, k, int(gated)))
+
+
 def mfma_alone(operands: torch.Tensor, workgroups: int, iters: int) -> float:
     """Runs the bfloat16 matrix instruction by itself on `operands` (at least
     32,768 bfloat16 values, held in registers) and returns the flop it did:

@@ -438,7 +438,12 @@ def test_gemm_tiled_weight(ops, n, m, k):
      # stages of 64 whose activations arrive as units of 8 tokens x 128 bytes: the last unit of
      # tokens partly empty, the last tile of k partly beyond k (its lanes fetch column 0)
      (1997, 3600, 424, False),
-     (500, 2048, 616, False)],   # tiles of 128 x 128, eight wavefronts
+     (500, 2048, 616, False),    # tiles of 128 x 128, eight wavefronts
+     # two products: the rows whose 256 x 256 tiles make a whole round of the compute
+     # units, then the rest with smaller tiles (gated pairs, a bias, rows that end
+     # inside a block of 16)
+     (500, 18950, 1024, True),
+     (500, 37900, 1024, False)],
 )
 def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
     """The large tiles with aligned rows and whole stages of k: operands go from
@@ -446,6 +451,7 @@ def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
     stages ends the ring of stage buffers at another place."""
     torch.manual_seed(21)
     dtype = torch.bfloat16
+    assert ops.gemm_parts(n, m, k, gated) == (2 if m > 18000 else 1)
     a = torch.randn(n, k)
     if gated:
         g, u = torch.randn(m, k) / math.sqrt(k) * 2, torch.randn(m, k) / math.sqrt(k)

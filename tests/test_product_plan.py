@@ -128,3 +128,19 @@ def test_shares_of_a_portions_keys():
     assert portion_splits(128, 1800) == 4 and portion_splits(256, 3600) == 2
     assert portion_splits(32, 8000) == 16 and portion_splits(4, 100000) == 64
     assert portion_splits(0, 5) == 1
+
+
+@pytest.mark.parametrize("gated", [False, True])
+@pytest.mark.parametrize("m, k", MATRICES)
+def test_a_product_in_two_parts_is_the_same_for_every_row_count_of_a_graph_bucket(m, k, gated):
+    """A product of many tokens may run as two (whole rounds of tiles, then the
+    rest): graphs of 128 and 256 rows must decide as every row count they stand for."""
+    for lo, hi in ((65, 128), (129, 256)):
+        assert len({ops.gemm_parts(n, m, k, gated) for n in range(lo, hi + 1)}) == 1
+    assert ops.gemm_parts(64, m, k, gated) == 1
+
+
+def test_where_a_product_runs_in_two_parts():
+    assert ops.gemm_parts(512, 18944, 3584, True) == 2    # 296 tiles of 256 x 256: 256 + 40
+    assert ops.gemm_parts(2048, 18944, 3584, True) == 1   # 1,184 tiles: the rest would take a round of its own anyway
+    assert ops.gemm_parts(512, 3584, 18944) == 1          # shares of k instead
