@@ -8,6 +8,7 @@ config.json chooses the model everywhere (engine, replay, command line).
 
 from __future__ import annotations
 
+import importlib
 import json
 import os
 from dataclasses import dataclass
@@ -50,7 +51,32 @@ def architectures() -> list[str]:
     return sorted(_ARCHITECTURES)
 
 
+_plugins_loaded = False
+
+
+def load_plugins() -> None:
+    """Imports what the environment variable SHRIKE_AMD_PLUGINS names, once:
+    comma-separated `module` or `module:function` entries.  A module registers
+    its architectures and parts when it is imported, or when `function()` is
+    called; that is how the command-line programs come to know an architecture
+    that is not part of the package."""
+    global _plugins_loaded
+    if _plugins_loaded:
+        return
+    _plugins_loaded = True
+    for entry in filter(None, (e.strip() for e in os.environ.get("SHRIKE_AMD_PLUGINS", "").split(","))):
+        module_name, _, function = entry.partition(":")
+        try:
+            module = importlib.import_module(module_name)
+            if function:
+                getattr(module, function)()
+        except Exception as e:
+            raise ConfigError(f"SHRIKE_AMD_PLUGINS: cannot load {entry!r}: {type(e).__name__}: {e}") from e
+
+
 def get_architecture(name: str) -> Architecture:
+    if name not in _ARCHITECTURES:
+        load_plugins()
     try:
         return _ARCHITECTURES[name]
     except KeyError:

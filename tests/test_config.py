@@ -154,3 +154,29 @@ def test_default_model_dir_env_override(monkeypatch):
     import shrike_amd.models.qwen2 as q
 
     importlib.reload(q)  # the reload emptied the registry; register again
+
+
+def test_plugins_named_in_the_environment_are_loaded_for_an_unknown_architecture(tmp_path, monkeypatch):
+    """SHRIKE_AMD_PLUGINS: how a program started from the command line learns an
+    architecture that is defined outside the package."""
+    import sys
+
+    from shrike_amd.config import registry
+
+    (tmp_path / "my_plugin.py").write_text(
+        "from shrike_amd.config.registry import register_architecture\n"
+        "from shrike_amd.models.qwen2 import Qwen2Config, build_spec\n"
+        "def install():\n"
+        "    register_architecture('PluggedInForCausalLM', Qwen2Config, build_spec)\n")
+    monkeypatch.syspath_prepend(str(tmp_path))
+    monkeypatch.setattr(registry, "_plugins_loaded", False)
+    monkeypatch.setenv("SHRIKE_AMD_PLUGINS", "my_plugin:install")
+    with pytest.raises(registry.ConfigError, match="unknown architecture"):
+        registry.get_architecture("NobodyForCausalLM")  # loads the plugins, still unknown
+    assert registry.get_architecture("PluggedInForCausalLM").config_cls.__name__ == "Qwen2Config"
+    registry._ARCHITECTURES.pop("PluggedInForCausalLM")
+    sys.modules.pop("my_plugin", None)
+    monkeypatch.setattr(registry, "_plugins_loaded", False)
+    monkeypatch.setenv("SHRIKE_AMD_PLUGINS", "no_such_module_anywhere")
+    with pytest.raises(registry.ConfigError, match="cannot load 'no_such_module_anywhere'"):
+        registry.get_architecture("NobodyForCausalLM")

@@ -4,14 +4,14 @@ tensor names, attention with an output bias, a rotation of part of each head
 and a scale that is not head_size**-0.5, and a schedule that runs the last
 layer twice (the second run with a cache of its own).  It is registered by
 name; the framework's writer makes its model folder, the Python entry point
-generates with it, bin/trace_run replays it, and a computation written out
-here with the plain functions checks both.  It is no model of anyone's: it
+generates with it, bin/trace_run replays it (told of this module by
+SHRIKE_AMD_PLUGINS), and a computation written out here with the plain
+functions checks both.  It is no model of anyone's: it
 shows that an architecture is added without a change to the framework's files."""
 
 import json
 import os
 import subprocess
-import sys
 from dataclasses import dataclass
 from pathlib import Path
 from typing import ClassVar
@@ -41,15 +41,6 @@ CONFIG = {
     "end_token": 210,
     "stored_as": "float32",
 }
-# how the module below is made known to bin/trace_run, which is another process
-PLUGIN = """
-import sys
-sys.path.insert(0, {repo!r})
-import tests.test_toy_architecture_gpu as toy
-toy.define()
-from shrike_amd.replay.trace import main
-sys.exit(main())
-"""
 
 
 @dataclass(frozen=True)
@@ -222,12 +213,11 @@ def test_the_toy_steps_and_generates_like_its_plain_form(toy, dtype, tol):
 
 
 def test_the_toy_through_trace_run(toy, tmp_path):
-    """bin/trace_run is another process: a three-line launcher imports this module,
-    registers the toy and hands over to the framework's own replay program."""
+    """bin/trace_run is another process: SHRIKE_AMD_PLUGINS names this module's
+    define(), which the registry calls when config.json names an architecture it
+    does not know."""
     folder, weights = toy
-    repo = str(Path(__file__).resolve().parent.parent)
-    launcher = tmp_path / "replay_toy.py"
-    launcher.write_text(PLUGIN.format(repo=repo))
+    repo = Path(__file__).resolve().parent.parent
     ids = torch.randint(0, 210, (30,), generator=torch.Generator().manual_seed(6)).tolist()
     steps = [
         {"step": 0, "entries": [{"id": "a", "tokens": ids[:19], "want": [0, 18]}], "end": []},
@@ -235,11 +225,12 @@ def test_the_toy_through_trace_run(toy, tmp_path):
         {"step": 2, "entries": [{"id": "a", "tokens": ids[29:], "want": [0]}], "end": ["a"]},
     ]
     out = tmp_path / "out"
+    env = dict(os.environ, SHRIKE_AMD_PLUGINS="tests.test_toy_architecture_gpu:define",
+               PYTHONPATH=os.pathsep.join(filter(None, [str(repo), os.environ.get("PYTHONPATH")])))
     proc = subprocess.run(
-        [sys.executable, str(launcher), "--model", str(folder), "--dtype", "float32", "--out", str(out),
+        [str(repo / "bin" / "trace_run"), "--model", str(folder), "--dtype", "float32", "--out", str(out),
          "--max-tokens", "64"],
-        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300,
-        env=dict(os.environ))
+        input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=300, env=env)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert [l for l in proc.stdout.splitlines() if l.startswith("done")] == ["done 0", "done 1", "done 2"]
     want = plain_logits(weights, ids)
