@@ -562,53 +562,6 @@ def test_toy_state_mixer_with_prepare_is_replayed_from_graphs():
         cache.free(s)
 
 
-def test_a_step_recorded_as_two_graphs_with_the_toy_state_mixer():
-    """Four schedule positions (both layers run twice, each run with a cache or a
-    state of its own): the decode step is recorded as two graphs, and the toy
-    mixer's state, which the first graph's run reads and the second's too, still
-    follows the recurrence."""
-    from shrike_amd.config.specs import ScheduleEntry
-    from shrike_amd.engine.runner import HEAD_BLOCKS
-
-    define_graph_safe_state_mixer()
-    base = small_spec()
-    toy_block = replace(base.blocks[1], mixer=DeviceDecaySpec(decay=0.6), mixer_name="decay")
-    order = (0, 1, 0, 1)
-    spec = replace(base, blocks=(base.blocks[0], toy_block), schedule=tuple(ScheduleEntry(b) for b in order))
-    assert len(order) >= 2 * HEAD_BLOCKS
-    w = cpu_weights(spec, seed=14)
-    runner, model, cache = make_runner(spec, w)
-    assert runner.use_graphs
-
-    def want_for(ids):
-        cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
-        wd = {k: v.double() for k, v in w.items()}
-        n = len(ids)
-        cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
-        x = wd["model.embed_tokens.weight"][torch.tensor(ids)]
-        p = "model.layers.1"
-        for block in order:
-            if block == 0:
-                x = plain.decoder_layer(cfg, wd, 0, x, cos, sin)
-                continue
-            u = plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5) @ wd[f"{p}.decay.in_proj.weight"].t()
-            state, ys = torch.zeros(48, dtype=torch.float64), []
-            for t in range(n):  # every run of the layer has a state of its own
-                state = 0.6 * state + u[t]
-                ys.append(state)
-            x = x + torch.stack(ys)
-            h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
-            x = x + plain.swiglu(h, wd[f"{p}.mlp.gate_proj.weight"], wd[f"{p}.mlp.up_proj.weight"],
-                                 wd[f"{p}.mlp.down_proj.weight"])
-        return plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
-
-    ids = torch.randint(0, 97, (30,), generator=torch.Generator().manual_seed(15)).tolist()
-    want = want_for(ids)
-    assert plain.rel_err(step_whole(runner, cache, ids, [6, 3] + [1] * 21), want) <= 1e-5
-    assert runner.graph_replays == 21
-    assert all(len(g.graphs) == 2 for g in runner._graphs.values())
-
-
 # ------------------------------------ a toy embedding and a toy head as parts of a model
 
 
