@@ -24,7 +24,6 @@ from .context import StepContext, StepShape, Workspace
 GRAPH_BATCH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 GRAPH_TABLE_QUANTUM = 64  # block-table widths of graphs are multiples of this
 MAX_GRAPHS = 24  # captured decode steps kept; the least recently used one goes first
-HEAD_BLOCKS = 2  # blocks in the first of a step's two recordings (see ModelRunner._record)
 
 
 @dataclass
@@ -78,7 +77,7 @@ class _DecodeGraph:
 
     def __init__(self, workspace: Workspace):
         self.workspace = workspace  # shared by the graphs of one batch bucket
-        self.graphs = []  # the step's recordings, replayed one after the other
+        self.graph = None
         self.meta_dev = None
         self.logits = None
         self.ctx = None
@@ -89,10 +88,6 @@ class _DecodeGraph:
         self.offsets = None  # field -> offset in the buffer; tables -> list of offsets
         self.rows = None  # the sequences of the last step, in row order
         self.table_lens = None  # per group, pages of each row already written to `host`
-
-    def replay(self) -> None:
-        for graph in self.graphs:
-            graph.replay()
 
 
 class ModelRunner:
@@ -305,7 +300,10 @@ class ModelRunner:
                 # now: a part that advances a state of its own must see each step once.
                 eager_logits = self.model.forward(g.ctx, self.layer_caches).clone()
                 torch.cuda.synchronize(self.runtime.device)
-                g.logits, g.graphs = self._record(g.ctx)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    g.logits = self.model.forward(g.ctx, self.layer_caches)
+                g.graph = graph
                 self._graphs[key] = g
                 self.graph_captures += 1
                 self.graph_replays += 1  # counted with the steps that the graph path served
@@ -314,39 +312,9 @@ class ModelRunner:
                 self._fill(g, entries, meta)
         g.meta_dev.copy_(g.pinned, non_blocking=True)
         g.copied.record()
-        g.replay()
+        g.graph.replay()
         self.graph_replays += 1
         return g.logits[: len(entries)]
-
-    def _record(self, ctx):
-        """Records the model's forward pass on `ctx` as HIP graphs: (logits, graphs).
-        Launching a graph of a few hundred kernels keeps the host busy for about
-        0.35 us a kernel before the device sees the first of them, so a model of
-        four layers or more is recorded as two graphs: a short one (embedding
-        and the first HEAD_BLOCKS layers), which starts within microseconds, and
-        the rest, whose launch the device does not wait for while it runs the first."""
-        split = HEAD_BLOCKS - 1 if len(self.model.spec.schedule) >= 2 * HEAD_BLOCKS else None
-        device = self.runtime.device
-        graphs = [torch.cuda.CUDAGraph()]
-        torch.cuda.synchronize(device)
-        current = torch.cuda.current_stream(device)
-        side = torch.cuda.Stream(device)
-        side.wait_stream(current)
-
-        def after_block(pos: int) -> None:
-            if pos == split:
-                graphs[-1].capture_end()
-                graphs.append(torch.cuda.CUDAGraph())
-                graphs[-1].capture_begin(pool=graphs[0].pool())
-
-        with torch.cuda.stream(side):
-            graphs[0].capture_begin()
-            try:
-                logits = self.model.forward(ctx, self.layer_caches, after_block=after_block)
-            finally:
-                graphs[-1].capture_end()
-        current.wait_stream(side)
-        return logits, graphs
 
     def _fill(self, g: _DecodeGraph, entries: list[StepEntry], meta: _Meta) -> None:
         """Writes a step's whole metadata into the graph's host buffer."""
@@ -422,7 +390,7 @@ class ModelRunner:
         g.host[off : off + n] = tokens
         g.meta_dev.copy_(g.pinned, non_blocking=True)
         g.copied.record()
-        g.replay()
+        g.graph.replay()
         self.graph_replays += 1
         for e in entries:
             e.cache.fresh_state = False

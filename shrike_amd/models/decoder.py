@@ -82,16 +82,12 @@ class DecoderModel:
         for part in self._preparers:
             part.prepare(shape)
 
-    def forward(self, ctx, caches, after_block=None) -> torch.Tensor:
+    def forward(self, ctx, caches) -> torch.Tensor:
         """Logits float32 [R, vocab] at ctx.out_rows.  `caches[i]` is the
-        LayerCache of schedule position i.  `after_block(pos)`, if given, is
-        called when schedule position `pos` has run (the runner ends one
-        recording there and begins the next)."""
+        LayerCache of schedule position i."""
         hidden = HiddenState(self.embedding.forward(ctx))
         for pos, entry in enumerate(self.spec.schedule):
             self.blocks[entry.block].forward(ctx, hidden, caches[pos])
-            if after_block is not None:
-                after_block(pos)
         rows = ctx.out_rows
         if rows.shape[0] == 0:
             return ctx.buffer("logits", (0, self.spec.vocab_size), torch.float32)
