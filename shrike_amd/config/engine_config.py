@@ -25,6 +25,10 @@ class EngineConfig:
     dtype: "bfloat16" (serving kernels) or "float32" (every kernel in true
         32-bit arithmetic); None takes the dtype the model folder was stored in.
     graphs: replay decode-only steps from HIP graphs.
+    overlap_steps: launch the next decode step before the host has read the
+        tokens of this one (they pass from the sampler to the next step on the
+        device); a request that turns out to have ended is dropped from that
+        step's results.
     """
 
     block_size: int = 16
@@ -36,6 +40,7 @@ class EngineConfig:
     dtype: str | None = None
     seed: int = 0
     graphs: bool = True
+    overlap_steps: bool = True
     device: str = "cuda:0"
 
     def __post_init__(self):

@@ -15,6 +15,12 @@ extern "C" {
 const char* shk_last_error(void);
 int shk_version(void);
 
+// dst[i] = src[i] for i < n, except dst[patch_at + j] = patch[j] for j < patch_n (patch
+// may be null with patch_n 0).  src and dst may be device memory or page-locked host
+// memory: small index arrays and tokens travel by this kernel, not by the copy engine.
+int shk_copy_words(const int32_t* src, int32_t* dst, int n, const int32_t* patch, int patch_at,
+                   int patch_n, void* stream);
+
 // out[i, :] = float(table[ids[i], :]); ids must lie in [0, vocab).
 int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int n, int hidden,
               int vocab, void* stream);

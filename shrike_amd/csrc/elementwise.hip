@@ -158,12 +158,37 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   out[row * inter + j] = from_float<T>(s * u);
 }
 
+// dst[i] = src[i], except dst[patch_at + j] = patch[j] for j < patch_n.  Either side
+// may be page-locked host memory: a step's index arrays come to the device, and
+// its chosen tokens go back, without the copy engine, whose hand-overs to and from
+// the compute queue cost more than these few hundred words.
+__global__ void __launch_bounds__(256)
+    copy_words_kernel(const int32_t* __restrict__ src, int32_t* __restrict__ dst, int n,
+                      const int32_t* __restrict__ patch, int patch_at, int patch_n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const int j = i - patch_at;
+  dst[i] = (j >= 0 && j < patch_n) ? patch[j] : src[i];
+}
+
 }  // namespace shk
 
 using namespace shk;
 
 extern "C" const char* shk_last_error(void) { return g_error; }
 extern "C" int shk_version(void) { return 1; }
+
+extern "C" int shk_copy_words(const int32_t* src, int32_t* dst, int n, const int32_t* patch,
+                              int patch_at, int patch_n, void* stream) {
+  SHK_REQUIRE(n >= 0 && patch_n >= 0 && patch_at >= 0 && patch_at + patch_n <= n,
+              "copy_words: bad sizes n=%d patch [%d, %d)", n, patch_at, patch_at + patch_n);
+  if (n == 0) return 0;
+  SHK_REQUIRE(src && dst && (patch || patch_n == 0), "copy_words: null pointer");
+  copy_words_kernel<<<(n + 255) / 256, 256, 0, static_cast<hipStream_t>(stream)>>>(src, dst, n, patch,
+                                                                                 patch_at, patch_n);
+  SHK_LAUNCH_CHECK("copy_words");
+  return 0;
+}
 
 extern "C" int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int n,
                          int hidden, int vocab, void* stream) {

@@ -16,7 +16,7 @@ from ..cache import CacheManager
 from ..config.engine_config import EngineConfig
 from ..sampling import Sampler
 from .loading import load_model
-from .request import Request, SamplingParams
+from .request import Request, SamplingParams, Status
 from .runner import ModelRunner, StepEntry
 from .scheduler import Scheduler
 
@@ -77,6 +77,9 @@ class LLMEngine:
         # (batch, prepared step) of the next step, laid out while the device ran the last
         # one; dropped whenever a request arrives, ends or is aborted
         self._planned = None
+        # (batch, logits) of a decode step that is already running on the device: it was
+        # launched, fed with the last step's tokens on the device, before the host read them
+        self._inflight = None
 
     # reference name for the cache manager
     @property
@@ -117,39 +120,60 @@ class LLMEngine:
         return self.scheduler.has_work
 
     def step(self) -> list[StepOutput]:
-        planned, self._planned = self._planned, None
-        running = self.scheduler.running
-        if planned is not None and (self.scheduler.waiting or len(planned[0]) != len(running)
-                                    or any(p[0] is not r for p, r in zip(planned[0], running))):
-            planned = None  # the queues were changed behind the engine's back
-        if planned is not None:
-            batch, prepared = planned
-        else:
-            batch, prepared = self.scheduler.schedule(), None
-        if not batch:
-            return []
-        entries, sampled = [], []
-        for req, n_new in batch:
-            start = req.num_computed_tokens
-            reaches_end = start + n_new >= req.num_tokens
-            entries.append(
-                StepEntry(req.cache, req.token_ids[start : start + n_new], start,
-                          [n_new - 1] if reaches_end else [])
-            )
-            if reaches_end:
-                sampled.append(req)
-        if prepared is not None:
-            logits = self.runner.launch_decode(prepared, [e.tokens[0] for e in entries])
-        else:
-            logits = self.runner.step(entries)
+        batch = logits = None
+        inflight, self._inflight = self._inflight, None
+        if inflight is not None:
+            # The step is already running.  Rows of requests that ended meanwhile
+            # (the end-of-sequence token, an abort) computed something nobody needs;
+            # what they wrote went into pages and slots that were theirs to write.
+            launched, all_logits = inflight
+            live = [i for i, (req, _) in enumerate(launched)
+                    if req.status is Status.RUNNING and self.requests.get(req.req_id) is req]
+            if live:
+                batch = [launched[i] for i in live]
+                logits = all_logits if len(live) == len(launched) else all_logits[
+                    torch.tensor(live, dtype=torch.long, device=all_logits.device)]
+                sampled = [req for req, _ in batch]
+        if batch is None:
+            planned, self._planned = self._planned, None
+            running = self.scheduler.running
+            if planned is not None and (self.scheduler.waiting or len(planned[0]) != len(running)
+                                        or any(p[0] is not r for p, r in zip(planned[0], running))):
+                planned = None  # the queues were changed behind the engine's back
+            if planned is not None:
+                batch, prepared = planned
+            else:
+                batch, prepared = self.scheduler.schedule(), None
+            if not batch:
+                return []
+            entries, sampled = [], []
+            for req, n_new in batch:
+                start = req.num_computed_tokens
+                reaches_end = start + n_new >= req.num_tokens
+                entries.append(
+                    StepEntry(req.cache, req.token_ids[start : start + n_new], start,
+                              [n_new - 1] if reaches_end else [])
+                )
+                if reaches_end:
+                    sampled.append(req)
+            if prepared is not None:
+                logits = self.runner.launch_decode(prepared, [e.tokens[0] for e in entries])
+            else:
+                logits = self.runner.step(entries)
         chosen = self.sampler.launch(logits, sampled)
 
         # While the device works: what does not depend on the tokens it will choose.
         self.scheduler.postprocess(batch)  # before finishing: finish() gives the pages back
         ahead = self.scheduler.plan_decode_step() if len(sampled) == len(batch) else None
         if ahead is not None:
-            self._planned = (ahead, self.runner.prepare_decode(
-                [req.cache for req, _ in ahead], [req.num_computed_tokens for req, _ in ahead]))
+            prepared = self.runner.prepare_decode(
+                [req.cache for req, _ in ahead], [req.num_computed_tokens for req, _ in ahead])
+            if (prepared is not None and self.config.overlap_steps and len(ahead) == len(sampled)
+                    and all(a[0] is r for a, r in zip(ahead, sampled))):
+                # the next step starts behind this one without waiting for the host
+                self._inflight = (ahead, self.runner.launch_decode_from(prepared, chosen.device))
+            else:
+                self._planned = (ahead, prepared)
 
         tokens = [] if chosen is None else chosen.tolist()  # waits for the device
         outputs: list[StepOutput] = []

@@ -19,6 +19,7 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, SequenceCache
+from ..kernels import ops
 from .context import StepContext, StepShape, Workspace
 
 GRAPH_BATCH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
@@ -291,7 +292,7 @@ class ModelRunner:
                     off += t.size
                 g.offsets = offsets
                 self._fill(g, entries, meta)
-                g.meta_dev.copy_(g.pinned, non_blocking=True)  # the eager run below reads it
+                ops.copy_words(g.pinned, g.meta_dev)  # the eager run below reads it
                 g.copied.record()
                 g.ctx = self._context(meta, g.meta_dev, g.workspace)
                 # This step itself runs kernel by kernel: every workspace buffer exists
@@ -310,7 +311,7 @@ class ModelRunner:
                 return eager_logits[: len(entries)]
             else:
                 self._fill(g, entries, meta)
-        g.meta_dev.copy_(g.pinned, non_blocking=True)
+        ops.copy_words(g.pinned, g.meta_dev)
         g.copied.record()
         g.graph.replay()
         self.graph_replays += 1
@@ -388,7 +389,24 @@ class ModelRunner:
             return self.step(entries)  # raises what an ordinary step raises
         off = g.offsets["token_ids"]
         g.host[off : off + n] = tokens
-        g.meta_dev.copy_(g.pinned, non_blocking=True)
+        ops.copy_words(g.pinned, g.meta_dev)
+        g.copied.record()
+        g.graph.replay()
+        self.graph_replays += 1
+        for e in entries:
+            e.cache.fresh_state = False
+        return g.logits[:n]
+
+    def launch_decode_from(self, prepared, tokens: torch.Tensor) -> torch.Tensor:
+        """launch_decode() with the tokens still on the device (int32, one per entry,
+        as the sampler of the step before left them): they are copied into the
+        step's metadata there, and the host need not know them to launch."""
+        g, entries = prepared
+        n = len(entries)
+        if tokens.dtype != torch.int32 or tokens.shape != (n,) or tokens.device != g.meta_dev.device:
+            raise ValueError("launch_decode_from: one int32 token per entry, on the model's device")
+        off = g.offsets["token_ids"]
+        ops.copy_words(g.pinned, g.meta_dev, patch=tokens, patch_at=off)
         g.copied.record()
         g.graph.replay()
         self.graph_replays += 1

@@ -58,6 +58,26 @@ class SplitSum:
         return self.parts.shape[1:]
 
 
+def _words(t: torch.Tensor, name: str) -> int:
+    """Address of an int32 tensor that a kernel may touch: on the device, or page-locked."""
+    if t.dtype != torch.int32 or not t.is_contiguous() or not (t.is_cuda or t.is_pinned()):
+        raise KernelError(f"{name}: expected a contiguous int32 tensor on the device or in page-locked memory")
+    return t.data_ptr()
+
+
+def copy_words(src: torch.Tensor, dst: torch.Tensor, patch: torch.Tensor | None = None, patch_at: int = 0) -> None:
+    """dst[:] = src[:] (int32, equal lengths) by a kernel, with dst[patch_at : patch_at +
+    len(patch)] taken from `patch` instead.  Either tensor may be page-locked host memory."""
+    n = src.numel()
+    if dst.numel() != n:
+        raise KernelError("copy_words: src and dst differ in length")
+    patch_n = 0 if patch is None else patch.numel()
+    if patch_at < 0 or patch_at + patch_n > n:
+        raise KernelError("copy_words: the patch does not fit")
+    check(load().shk_copy_words(_words(src, "src"), _words(dst, "dst"), n,
+                                None if patch is None else _words(patch, "patch"), patch_at, patch_n, _stream()))
+
+
 def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
     """out[i] = float(table[ids[i]]); ids int32 [n], out float32 [n, hidden]."""
     n, hidden = out.shape

@@ -29,6 +29,20 @@ def uniform(seed: int, draw: int) -> float:
     return (splitmix64(splitmix64(seed & _MASK) ^ (draw & _MASK)) >> 40) / float(1 << 24)
 
 
+class ChosenTokens:
+    """The tokens of a step, on the device (`device`, int32) and on their way to
+    the host: the copy into page-locked memory is queued right behind the
+    kernel that chose them, ahead of whatever is launched next, and tolist()
+    waits for that copy alone."""
+
+    def __init__(self, device: torch.Tensor, host: torch.Tensor, copied: torch.cuda.Event):
+        self.device, self._host, self._copied = device, host, copied
+
+    def tolist(self) -> list[int]:
+        self._copied.synchronize()
+        return self._host.tolist()
+
+
 class Sampler:
     def __init__(self, device, engine_seed: int = 0):
         self.device = device
@@ -40,17 +54,26 @@ class Sampler:
             return req.sampling.seed
         return splitmix64((self.engine_seed << 20) ^ req.req_id)
 
-    def launch(self, logits: torch.Tensor, reqs: list) -> torch.Tensor | None:
+    def launch(self, logits: torch.Tensor, reqs: list) -> ChosenTokens | None:
         """Starts the choice of one token per row of logits (float32 [R, vocab]
-        on the device, one row per request) and returns the device tensor that
-        will hold them; nothing here waits for the device."""
+        on the device, one row per request) and their copy to the host; returns
+        the handle that holds them.  Nothing here waits for the device."""
         if not reqs:
             return None
-        rows, vocab = logits.shape
+        rows = logits.shape[0]
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
+        self._choose(logits, out, reqs)
+        host = torch.empty(rows, dtype=torch.int32, pin_memory=True)
+        ops.copy_words(out, host)
+        copied = torch.cuda.Event()
+        copied.record()
+        return ChosenTokens(out, host, copied)
+
+    def _choose(self, logits: torch.Tensor, out: torch.Tensor, reqs: list) -> None:
+        rows, vocab = logits.shape
         if all(r.sampling.temperature == 0.0 for r in reqs):
             ops.argmax(logits, out)
-            return out
+            return
         params = torch.tensor(
             [[r.sampling.temperature for r in reqs],
              [r.sampling.top_p for r in reqs],
@@ -60,7 +83,6 @@ class Sampler:
         if self._scratch is None or self._scratch.numel() < rows * vocab:
             self._scratch = torch.empty(rows * vocab, dtype=torch.float32, device=logits.device)
         ops.sample(logits, out, params[0], params[1], params[2], self._scratch)
-        return out
 
     def sample(self, logits: torch.Tensor, reqs: list) -> list[int]:
         """The tokens themselves: launch(), then the wait for the device."""

@@ -220,6 +220,54 @@ def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol):
     cache.check([])
 
 
+def test_overlapped_steps_change_no_token(model_root, tmp_path):
+    """The next decode step is launched before the host has read this step's tokens.
+    With a fifth of all token ids ending a sequence, requests end at steps that
+    nobody can foresee, and some are aborted while a step that holds them is
+    already running: every request still yields exactly what an engine that does
+    not overlap yields for it alone, greedy or drawn."""
+    from shrike_amd import SamplingParams
+    from shrike_amd.engine.llm_engine import LLMEngine
+    from shrike_amd.weights import write_model_folder
+
+    cfg = dict(CONFIGS["B"], eos_token_id=list(range(3, CONFIGS["B"]["vocab_size"], 5)))
+    model_dir = write_model_folder(cfg, tmp_path / "many_ends", seed=5, mode="unit")
+    rng = random.Random(21)
+    jobs = []
+    for i in range(24):
+        prompt = prompts_for("B", [rng.randint(1, 40)], seed=300 + i)[0]
+        jobs.append((prompt, SamplingParams(max_new_tokens=rng.randint(1, 40), top_p=0.95, seed=i,
+                                            temperature=0.0 if i % 3 else 0.9)))
+    alone = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64,
+                      enable_prefix_caching=False, overlap_steps=False)
+    want = [alone.generate([p], sp)[0] for p, sp in jobs]
+    assert 4 < sum(len(w) < sp.max_new_tokens for w, (_, sp) in zip(want, jobs)) < 24
+
+    engine = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=80, max_running=8)
+    assert engine.config.overlap_steps
+    got, ids, pending, aborted, overlapped = {}, {}, list(range(len(jobs))), set(), 0
+    while pending or engine.has_work:
+        for _ in range(8 if len(pending) == len(jobs) else int(rng.random() < 0.3)):
+            if pending:  # eight requests to begin with, then one now and then
+                i = pending.pop(0)
+                ids[engine.add_request(jobs[i][0], jobs[i][1])] = i
+        if engine._inflight is not None:
+            overlapped += 1
+            if len(aborted) < 3 and rng.random() < 0.3:  # a request of the step that is running
+                victim = rng.choice(engine._inflight[0])[0]
+                aborted.add(ids[victim.req_id])
+                engine.abort(victim.req_id)
+        for o in engine.step():
+            got.setdefault(ids[o.req_id], []).append(o.token_id)
+        engine.cache.check([r.cache for r in engine.scheduler.running if r.cache is not None])
+    assert overlapped > 10 and aborted
+    for i, w in enumerate(want):
+        mine = got.get(i, [])
+        assert mine == (w[: len(mine)] if i in aborted else w), f"request {i}"
+    assert engine.cache.num_free == 80 and not engine.scheduler.running
+    engine.cache.check([])
+
+
 def test_add_request_guards(model_root):
     # tests/test_review_regressions.py:90-93
     from shrike_amd import SamplingParams

@@ -475,6 +475,30 @@ def test_large_products_that_load_straight_into_lds(ops, n, m, k, gated):
     assert torch.equal(part, out[first : first + 300])
 
 
+def test_copy_words_between_page_locked_and_device_memory(ops):
+    """The kernel that carries a step's index arrays to the device and its tokens
+    back, with the tokens of the step before patched in on the way."""
+    from shrike_amd.kernels.ops import KernelError
+
+    host = torch.arange(1000, dtype=torch.int32).pin_memory()
+    dev_buf = torch.full((1000,), -1, dtype=torch.int32, device="cuda")
+    ops.copy_words(host, dev_buf)
+    assert torch.equal(dev_buf.cpu(), host)
+    patch = torch.tensor([7, 8, 9], dtype=torch.int32, device="cuda")
+    ops.copy_words(host, dev_buf, patch=patch, patch_at=997)
+    want = host.clone()
+    want[997:] = torch.tensor([7, 8, 9], dtype=torch.int32)
+    assert torch.equal(dev_buf.cpu(), want)
+    back = torch.zeros(1000, dtype=torch.int32).pin_memory()
+    ops.copy_words(dev_buf, back)
+    torch.cuda.synchronize()
+    assert torch.equal(back, want)
+    with pytest.raises(KernelError):
+        ops.copy_words(host, dev_buf, patch=patch, patch_at=998)  # the patch does not fit
+    with pytest.raises(KernelError):
+        ops.copy_words(torch.arange(1000, dtype=torch.int32), dev_buf)  # pageable host memory
+
+
 def test_matrix_units_alone(ops):
     """The measuring kernel behind the benchmark's `mfma_tflops`: it runs, says how
     many flop it did, and refuses operands that would be read out of bounds."""
