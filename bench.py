@@ -289,17 +289,17 @@ def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
         engine.step()
     torch.cuda.synchronize()
     decode_ms = (time.perf_counter() - t0) / 50 * 1e3
-    engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)],
-                       SamplingParams(max_new_tokens=8, ignore_eos=True))
+    late = engine.requests[engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)],
+                                              SamplingParams(max_new_tokens=8, ignore_eos=True))]
     full = []  # steps that use the whole budget
     while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
-        left = max(r.num_tokens - r.num_computed_tokens for r in list(engine.scheduler.waiting) +
-                   engine.scheduler.running)
+        done = late.num_computed_tokens
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         engine.step()
         torch.cuda.synchronize()
-        if left >= budget - decodes:
+        # (a decode step that was already running when the prompt arrived is not one of them)
+        if late.num_computed_tokens - done >= budget - decodes:
             full.append((time.perf_counter() - t0) * 1e3)
     for req in list(engine.scheduler.running):
         engine.abort(req.req_id)
