@@ -309,6 +309,7 @@ def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
 
 
 def main() -> int:
+    global CONTEXT_END
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
     ap.add_argument("--steps", type=int, default=1900,
@@ -320,6 +321,9 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--context", type=int, default=PROMPT_LEN, metavar="N",
                     help="start decoding at a context of N tokens (N-token prompts) instead of 2,048")
+    ap.add_argument("--context-end", type=int, default=CONTEXT_END, metavar="N",
+                    help="the context length the cache is made for (the configuration's 4,096; more for runs "
+                         "at longer contexts)")
     ap.add_argument("--far-context", type=int, default=4000 - 64, metavar="N",
                     help="context of the extra points decode_b*_ctx4000 (0: leave them out)")
     ap.add_argument("--no-peaks", action="store_true",
@@ -337,6 +341,7 @@ def main() -> int:
     if args.steps < 1 or args.warmup < 0 or args.batch < 1:
         print("bench.py: --steps and --batch must be positive, --warmup non-negative")
         return 2
+    CONTEXT_END = args.context_end
     if not 1 <= args.context < CONTEXT_END:
         print(f"bench.py: --context must lie in [1, {CONTEXT_END})")
         return 2
