@@ -40,6 +40,9 @@ def parse_args(argv=None) -> argparse.Namespace:
     ap.add_argument("--max-tokens-per-step", type=int, default=512)
     ap.add_argument("--max-running", type=int, default=256)
     ap.add_argument("--no-prefix-caching", action="store_true")
+    ap.add_argument("--no-graphs", action="store_true", help="run decode steps kernel by kernel")
+    ap.add_argument("--no-overlap", action="store_true",
+                    help="launch a decode step only when the tokens of the step before are on the host")
     ap.add_argument("--metrics", action="store_true", help="print engine metrics at the end")
     return ap.parse_args(argv)
 
@@ -53,7 +56,7 @@ def main(argv=None) -> int:
         block_size=args.block_size, gpu_mem_util=args.gpu_mem_util,
         max_tokens_per_step=args.max_tokens_per_step, max_running=args.max_running,
         enable_prefix_caching=not args.no_prefix_caching, num_kv_blocks=args.num_kv_blocks,
-        dtype=args.dtype, seed=args.seed,
+        dtype=args.dtype, seed=args.seed, graphs=not args.no_graphs, overlap_steps=not args.no_overlap,
     )
     if args.random_config is not None:
         import json
