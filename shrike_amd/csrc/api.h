@@ -116,11 +116,13 @@ int shk_attention_supports_mfma(int heads, int kv_heads, int head_dim, int page_
 // bfloat16 decode attention: sequence s has one query token, row s of q, at
 // positions[s].  Its keys are split over nsplit wavefronts per key/value head;
 // `partial` is float32 scratch of num_seqs * heads * nsplit * (head_dim + 2).
+// streaming != 0: keys and values are fetched with non-temporal loads (faster when a
+// launch reads tens of megabytes of them, slightly slower below; the result is the same).
 int shk_attention_decode_bf16(const void* q, int q_stride, void* out, int num_seqs, int heads,
                               int kv_heads, int head_dim, const int32_t* positions,
                               const int32_t* tables, int table_stride, const void* k_pool,
                               const void* v_pool, int page_size, int window, float scale,
-                              float* partial, int nsplit, void* stream);
+                              float* partial, int nsplit, int streaming, void* stream);
 
 // bfloat16 attention for prompt portions, in tiles of 16 queries: tile i covers
 // queries tile_q0[i] .. +16 of sequence tile_seq[i]'s portion.  cu_q[s] is the

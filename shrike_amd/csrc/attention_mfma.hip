@@ -290,6 +290,12 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
 //                 element: one 16-byte load from the transposed page).
 // Keys outside [lo, pos] are loaded from a slot of a page the sequence holds
 // (the page of the nearest key inside the range) and masked.
+//
+// NT: keys and values are fetched with non-temporal loads.  Nothing is read twice
+// within a launch, and from some 50 MB of keys and values per launch on the stream
+// then runs a tenth faster (64 sequences of 2,200 keys: 49.7 us against 54.1; of
+// 4,000: 86.0 against 95.4, 6.1 TB/s); below that size it is 1 to 4 % slower, so
+// the caller says which it wants.
 
 constexpr int kMaxSplits = 64;
 constexpr int kDecodeWaves = 4;
@@ -316,7 +322,7 @@ struct PageDiv {
   __device__ __forceinline__ int mod(int x) const { return x - div(x) * ps; }
 };
 
-template <int D>
+template <int D, bool NT>
 __global__ void __launch_bounds__(kDecodeWaves* kWave)
     attention_decode_kernel(const bf16* __restrict__ q, int q_stride, bf16* __restrict__ out,
                             int heads, int kv_heads, const int32_t* __restrict__ positions,
@@ -392,12 +398,16 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int ds = 0; ds < D / 32; ++ds)
-          c.k[t][ds].u = *reinterpret_cast<const uint4*>(krow + k_lane[t] +
-                                                         static_cast<size_t>(ds) * page_size * 32);
+          c.k[t][ds].v = NT ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(
+                                  krow + k_lane[t] + static_cast<size_t>(ds) * page_size * 32))
+                            : *reinterpret_cast<const bf16x8*>(krow + k_lane[t] +
+                                                              static_cast<size_t>(ds) * page_size * 32);
       const bf16* vcol = v_pool + (v_second ? head_c + slot_c : head_a + slot_a) + v_lane;
 #pragma unroll
       for (int db = 0; db < D / 16; ++db)
-        c.v[db].u = *reinterpret_cast<const uint4*>(vcol + static_cast<size_t>(db) * 16 * page_size);
+        c.v[db].v = NT ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(
+                             vcol + static_cast<size_t>(db) * 16 * page_size))
+                       : *reinterpret_cast<const bf16x8*>(vcol + static_cast<size_t>(db) * 16 * page_size);
     };
 
     auto attend_chunk = [&](const DecodeChunk<D>& c, int kb, auto edge_tag) {
@@ -972,11 +982,16 @@ template <int D>
 static void launch_decode(dim3 grid, hipStream_t s, const bf16* q, int q_stride, bf16* out,
                           int heads, int kv_heads, const int32_t* positions, const int32_t* tables,
                           int table_stride, const bf16* k_pool, const bf16* v_pool, int page_size,
-                          int window, float scale, float* partial, int nsplit) {
+                          int window, float scale, float* partial, int nsplit, int streaming) {
   const uint32_t magic = static_cast<uint32_t>(((1ull << 32) + page_size - 1) / page_size);
-  attention_decode_kernel<D><<<grid, kDecodeWaves * kWave, 0, s>>>(q, q_stride, out, heads, kv_heads, positions,
-                                                    tables, table_stride, k_pool, v_pool, page_size,
-                                                    magic, window, scale, partial, nsplit);
+  if (streaming)
+    attention_decode_kernel<D, true><<<grid, kDecodeWaves * kWave, 0, s>>>(
+        q, q_stride, out, heads, kv_heads, positions, tables, table_stride, k_pool, v_pool, page_size,
+        magic, window, scale, partial, nsplit);
+  else
+    attention_decode_kernel<D, false><<<grid, kDecodeWaves * kWave, 0, s>>>(
+        q, q_stride, out, heads, kv_heads, positions, tables, table_stride, k_pool, v_pool, page_size,
+        magic, window, scale, partial, nsplit);
   if (nsplit > 1)
     attention_merge_kernel<D><<<grid.y * heads, kWave, 0, s>>>(partial, out, nsplit);
 }
@@ -1059,7 +1074,7 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
                                          const int32_t* positions, const int32_t* tables,
                                          int table_stride, const void* k_pool, const void* v_pool,
                                          int page_size, int window, float scale, float* partial,
-                                         int nsplit, void* stream) {
+                                         int nsplit, int streaming, void* stream) {
   if (check_mfma_shapes("attention_decode", heads, kv_heads, head_dim, page_size, q_stride)) return 1;
   SHK_REQUIRE(heads / kv_heads <= 16, "attention_decode: at most 16 query heads per key/value head");
   SHK_REQUIRE(num_seqs >= 0 && num_seqs <= 65535 && nsplit >= 1 && nsplit <= kMaxSplits,
@@ -1079,7 +1094,8 @@ extern "C" int shk_attention_decode_bf16(const void* q, int q_stride, void* out,
 #define CALL(D)                                                                              \
   launch_decode<D>(grid, s, static_cast<const bf16*>(q), q_stride, static_cast<bf16*>(out), heads, \
                    kv_heads, positions, tables, table_stride, static_cast<const bf16*>(k_pool),    \
-                   static_cast<const bf16*>(v_pool), page_size, window, scale, partial, nsplit)
+                   static_cast<const bf16*>(v_pool), page_size, window, scale, partial, nsplit,    \
+                   streaming)
   SHK_DISPATCH_D(head_dim, CALL)
 #undef CALL
   SHK_LAUNCH_CHECK("attention_decode");

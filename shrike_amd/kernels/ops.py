@@ -331,8 +331,10 @@ def attention_supports_mfma(heads, kv_heads, head_dim, page_size, q_stride) -> b
 
 
 def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tables, k_pool, v_pool,
-                     page_size, window, scale, partial, nsplit) -> None:
-    """bfloat16 MFMA attention for the first num_seqs rows of q, one token per sequence."""
+                     page_size, window, scale, partial, nsplit, streaming=False) -> None:
+    """bfloat16 MFMA attention for the first num_seqs rows of q, one token per sequence.
+    `streaming`: fetch keys and values with non-temporal loads (same result; faster when
+    the launch reads tens of megabytes of them)."""
     _rows(q, "attention_decode q")
     if q.dtype != torch.bfloat16 or out.dtype != torch.bfloat16:
         raise KernelError("attention_decode: bfloat16 only")
@@ -349,7 +351,7 @@ def attention_decode(q, out, num_seqs, heads, kv_heads, head_dim, positions, tab
             _dev(positions, "positions", torch.int32), _dev(tables, "tables", torch.int32),
             tables.shape[1], _dev(k_pool, "k_pool"), _dev(v_pool, "v_pool"), page_size,
             int(window or 0), float(scale), _dev(partial, "partial", torch.float32), nsplit,
-            _stream(),
+            int(bool(streaming)), _stream(),
         )
     )
 

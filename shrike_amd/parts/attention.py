@@ -14,6 +14,9 @@ QUERY_TILE = 16  # queries per tile of the MFMA kernels for prompt portions
 COMPUTE_UNITS = 256
 KEYS_PER_WORKGROUP = 256  # a decode workgroup's four wavefronts want at least this many keys
 MAX_KEY_SPLITS = 64
+# decode attention fetches keys and values with non-temporal loads from this many bytes
+# of them per launch on (counted with the batch and the context rounded up to powers of two)
+STREAMING_FROM_BYTES = 96 << 20
 # prompt portions take workgroups of 8 wavefronts instead of 16 while no more than this many
 # of them are launched: two fit on a compute unit, so all of them run at once
 SMALL_WORKGROUPS_AT_ONCE = 2 * COMPUTE_UNITS
@@ -37,12 +40,25 @@ def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
     return max(1, min(want, most, MAX_KEY_SPLITS))
 
 
+def decode_streams(num_seqs: int, kv_heads: int, head_dim: int, max_ctx: int, window: int | None = None) -> bool:
+    """Whether a decode launch reads so many keys and values that non-temporal
+    loads pay (measured with 4 key/value heads of 128: a tenth faster from 64
+    sequences of 2,200 keys or 8 of 16,000, 2 % at 8 of 4,000, 1 to 4 % slower
+    below).  The result is the same either way; batch and context are rounded up
+    as in decode_splits(), so that a graph's steps all decide alike."""
+    keys = _pow2(max_ctx, KEYS_PER_WORKGROUP)
+    if window:
+        keys = min(keys, window)
+    return _pow2(num_seqs) * keys * kv_heads * head_dim * 4 >= STREAMING_FROM_BYTES
+
+
 @dataclass
 class AttentionPlan:
     """How one step's attention is launched for a (heads, kv heads, head size)."""
 
     mfma: bool = False
     nsplit: int = 1  # key splits of the single-token rows
+    streaming: bool = False  # single-token rows: non-temporal loads of keys and values
     kernel: str = ""  # for prompt portions: "shared", "tiles" or "" (none in the step)
     small: bool = False  # "shared" with half as many wavefronts per workgroup
     portion_splits: int = 1  # "shared": workgroups that share an entry's keys
@@ -179,7 +195,8 @@ class PagedAttention(Mixer):
             return  # the general kernel takes every token alike
         if shape.num_decode:
             plan.nsplit = decode_splits(shape.num_decode, hkv, shape.max_decode_ctx)
-            shape.launch_key.append((key, plan.nsplit))
+            plan.streaming = decode_streams(shape.num_decode, hkv, d, shape.max_decode_ctx, s.window)
+            shape.launch_key.append((key, plan.nsplit, plan.streaming))
         portions = shape.q_lens[shape.num_decode:]
         if portions.size == 0:
             return
@@ -231,7 +248,7 @@ class PagedAttention(Mixer):
                                  torch.float32)
             ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
                                  cache.k_pool, cache.v_pool, cache.page_size, s.window, s.scale,
-                                 partial, plan.nsplit)
+                                 partial, plan.nsplit, plan.streaming)
         if plan.kernel == "shared":
             partial = None
             if plan.portion_splits > 1:

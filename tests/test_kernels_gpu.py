@@ -567,6 +567,12 @@ def test_attention_decode_mfma(ops, heads, kv_heads, head_dim, page_size, window
     want = reference_attention(q.double(), k_pool, v_pool, tables, [1] * n, [c - 1 for c in ctx], page_size, window, scale)
     assert not torch.isnan(out.float()).any(), "a slot outside the context reached the output"
     close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
+    # with non-temporal loads of keys and values: the same bits
+    streamed = torch.full_like(out, float("nan"))
+    partial.fill_(float("nan"))
+    ops.attention_decode(dev(q).view(n, -1), streamed, n, heads, kv_heads, head_dim, dev(positions), tables,
+                         k_pool, v_pool, page_size, window, scale, partial, nsplit, streaming=True)
+    assert torch.equal(streamed, out)
 
 
 @pytest.mark.parametrize(
@@ -922,7 +928,7 @@ def test_attention_decode_finds_far_keys_in_a_long_context(ops, ctx, special):
         out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
         partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
         ops.attention_decode(dev(q.to(dtype)).view(n, -1), out, n, heads, kv_heads, head_dim, dev(positions), tables,
-                             k_pool, v_pool, page_size, None, scale, partial, nsplit)
+                             k_pool, v_pool, page_size, None, scale, partial, nsplit, streaming=nsplit > 1)
         want = reference_attention(q.to(dtype).double(), k_pool, v_pool, tables, [1] * n, [c - 1 for c in ctx],
                                    page_size, None, scale)
         got = out.view(n, heads, head_dim)

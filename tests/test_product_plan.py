@@ -51,6 +51,19 @@ def test_key_splits_of_decode_attention_depend_on_the_buckets_only():
     assert decode_splits(8, 4, 2100) == 8 and decode_splits(64, 4, 4000) == 1 and decode_splits(1, 4, 100) == 1
 
 
+def test_non_temporal_loads_from_a_size_on_and_alike_within_a_bucket():
+    from shrike_amd.parts.attention import decode_streams
+
+    # 7B heads: 8 sequences at 2,100 keys stay as they were, 64 of them or 8 at 16,000 stream
+    assert not decode_streams(8, 4, 128, 2100) and not decode_streams(1, 4, 128, 4000)
+    assert decode_streams(64, 4, 128, 2100) and decode_streams(8, 4, 128, 16000) and decode_streams(16, 4, 128, 2100)
+    # a window bounds what is read
+    assert not decode_streams(64, 4, 128, 100000, window=256)
+    for seqs_lo, seqs_hi in ((3, 4), (5, 8), (33, 64), (129, 256)):
+        for ctx_lo, ctx_hi in ((257, 512), (2049, 4096), (16385, 32768)):
+            assert len({decode_streams(s, 4, 128, c) for s in (seqs_lo, seqs_hi) for c in (ctx_lo, ctx_hi)}) == 1
+
+
 def test_decode_graphs_are_keyed_by_buckets_and_few():
     """The key of a decode graph: batch bucket, table widths in steps of 64
     pages, and what the parts' launches depend on (here the split of the keys).
