@@ -181,14 +181,24 @@ def test_long_decoding_and_first_tokens(model_root):
         cache.check([])
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
-def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol):
+@pytest.mark.parametrize("dtype, tol, streamed", [("float32", 1e-4, False), ("bfloat16", 3e-2, False),
+                                                  ("bfloat16", 3e-2, True)])
+def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol, streamed, monkeypatch):
     """A 10,000-token prompt in portions of up to 4,096 tokens (the later ones
     read keys far back, through block tables of more than 600 pages), then six
-    single tokens from a graph with the key splits the engine chooses there."""
+    single tokens from a graph with the key splits the engine chooses there;
+    `streamed`: with the non-temporal loads that the engine takes for large batches."""
     from shrike_amd.cache import CacheManager
     from shrike_amd.engine.loading import load_model
     from shrike_amd.engine.runner import ModelRunner, StepEntry
+    from shrike_amd.kernels import ops
+    from shrike_amd.parts import attention
+
+    if streamed:
+        monkeypatch.setattr(attention, "STREAMING_FROM_BYTES", 0)
+    flags = []
+    launch = ops.attention_decode
+    monkeypatch.setattr(ops, "attention_decode", lambda *a: (flags.append(a[15]), launch(*a))[1])
 
     model_dir = make_model_dir("B", model_root, dtype=dtype, mode="unit")
     ids = prompts_for("B", [10006], seed=9)[0]
@@ -212,6 +222,7 @@ def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol):
         cache.append(seq, p, 1)
         got.append(runner.step([StepEntry(seq, [ids[p]], p, [0])]).cpu().double())
     assert runner.graph_replays == 6
+    assert flags and all(f == streamed for f in flags) if dtype == "bfloat16" else not flags
     got = torch.cat(got)
     assert torch.isfinite(got).all()
     err = (got - want).abs().amax(-1) / want.abs().max()
