@@ -178,9 +178,13 @@ int shk_argmax_static_max_floats(void);
 
 // Temperature / top-p sampling of one token per row (see sampling.hip).
 // temperature[r] == 0 takes the argmax.  uniforms[r] in [0, 1) is the draw.
-// `scratch` is float32 [rows, vocab].
+// `scratch` holds scratch_floats >= shk_sample_scratch_floats(rows, vocab) floats,
+// 16-byte aligned.  nucleus == 0 promises that every row's top_p is 1 or more
+// (the passes that find the nucleus are then left out; top_p is not read).
 int shk_sample(const float* logits, int32_t* out, const float* temperature, const float* top_p,
-               const float* uniforms, float* scratch, int rows, int vocab, int ld, void* stream);
+               const float* uniforms, float* scratch, long long scratch_floats, int rows, int vocab,
+               int ld, int nucleus, void* stream);
+long long shk_sample_scratch_floats(int rows, int vocab);
 
 #ifdef __cplusplus
 }

@@ -5,7 +5,7 @@ in the product path runs."""
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 _LIB = None
 
@@ -38,7 +38,7 @@ _SIGNATURES = {
                                           _P, _I, _I, _I, _P],
     "shk_argmax": [_P, _P, _I, _I, _I, _P, _P],
     "shk_argmax_scratch_floats": [_I, _I],
-    "shk_sample": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "shk_sample": [_P, _P, _P, _P, _P, _P, c_longlong, _I, _I, _I, _I, _P],
 }
 
 
@@ -57,6 +57,8 @@ def load():
             fn = getattr(lib, name)
             fn.argtypes = argtypes
             fn.restype = c_int
+        lib.shk_sample_scratch_floats.argtypes = [_I, _I]
+        lib.shk_sample_scratch_floats.restype = c_longlong
         lib._path = str(path)
         _LIB = lib
     return _LIB

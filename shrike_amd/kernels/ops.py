@@ -440,17 +440,24 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
                             None if scratch is None else scratch.data_ptr(), _stream()))
 
 
-def sample(logits, out, temperature, top_p, uniforms, scratch) -> None:
-    """One token per row: argmax where temperature is 0, else a top-p draw with uniforms[r]."""
+def sample_scratch_floats(rows: int, vocab: int) -> int:
+    """float32 elements of scratch that sample() needs for logits [rows, vocab]."""
+    return int(load().shk_sample_scratch_floats(rows, vocab))
+
+
+def sample(logits, out, temperature, top_p, uniforms, scratch, nucleus: bool = True) -> None:
+    """One token per row: argmax where temperature is 0, else a top-p draw with uniforms[r].
+    nucleus=False promises that no row has a top_p below 1 (fewer passes)."""
     _rows(logits, "sample logits")
     rows, vocab = logits.shape
-    if scratch.numel() < rows * vocab:
-        raise KernelError("sample: scratch needs rows * vocab float32 elements")
+    if scratch.numel() < sample_scratch_floats(rows, vocab):
+        raise KernelError(f"sample: scratch needs {sample_scratch_floats(rows, vocab)} float32 elements "
+                          "(sample_scratch_floats)")
     check(
         load().shk_sample(
             _dev(logits, "logits", torch.float32), _dev(out, "out", torch.int32),
             _dev(temperature, "temperature", torch.float32), _dev(top_p, "top_p", torch.float32),
             _dev(uniforms, "uniforms", torch.float32), _dev(scratch, "scratch", torch.float32),
-            rows, vocab, logits.stride(0), _stream(),
+            scratch.numel(), rows, vocab, logits.stride(0), int(bool(nucleus)), _stream(),
         )
     )

@@ -80,9 +80,11 @@ class Sampler:
              [uniform(self.request_seed(r), r.num_generated) for r in reqs]],
             dtype=torch.float32,
         ).to(logits.device)
-        if self._scratch is None or self._scratch.numel() < rows * vocab:
-            self._scratch = torch.empty(rows * vocab, dtype=torch.float32, device=logits.device)
-        ops.sample(logits, out, params[0], params[1], params[2], self._scratch)
+        need = ops.sample_scratch_floats(rows, vocab)
+        if self._scratch is None or self._scratch.numel() < need:
+            self._scratch = torch.empty(need, dtype=torch.float32, device=logits.device)
+        nucleus = any(r.sampling.temperature > 0.0 and r.sampling.top_p < 1.0 for r in reqs)
+        ops.sample(logits, out, params[0], params[1], params[2], self._scratch, nucleus=nucleus)
 
     def sample(self, logits: torch.Tensor, reqs: list) -> list[int]:
         """The tokens themselves: launch(), then the wait for the device."""

@@ -334,11 +334,12 @@ def test_argmax_takes_the_lowest_index_among_equal_maxima(ops):
     assert out2.tolist() == [1, 0]
 
 
-def run_sample(ops, logits, temperature, top_p, u):
+def run_sample(ops, logits, temperature, top_p, u, nucleus=True):
     rows, vocab = logits.shape
-    out = torch.empty(rows, dtype=torch.int32, device="cuda")
+    out = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
     f = lambda x: torch.tensor(x, dtype=torch.float32, device="cuda")  # noqa: E731
-    ops.sample(dev(logits), out, f(temperature), f(top_p), f(u), torch.empty(rows * vocab, device="cuda"))
+    scratch = torch.full((ops.sample_scratch_floats(rows, vocab),), float("nan"), device="cuda")
+    ops.sample(dev(logits), out, f(temperature), f(top_p), f(u), scratch, nucleus=nucleus)
     return out.tolist()
 
 
@@ -378,6 +379,66 @@ def test_sample_keeps_as_many_equal_weights_as_the_rule_admits(ops):
     for u in [i / 40 for i in range(40)]:
         got.update(run_sample(ops, logits, [1.0], [0.35], [u]))
     assert got == {0, 1, 2, 3}
+
+
+def test_sample_over_the_vocabulary_of_the_7b_model(ops):
+    """152,064 logits are 38 chunks of 4096: the kept set is the plain rule's and the
+    draw the inverse of the cumulative kept weight in index order, whatever chunk it
+    falls in; rows of every kind side by side (greedy, no nucleus, narrow and wide ones)."""
+    torch.manual_seed(17)
+    vocab = 152064
+    base = torch.randn(vocab) * 3
+    cases = [(0.0, 1.0), (1.0, 1.0), (0.7, 0.9), (1.5, 0.3), (0.2, 0.05), (1.0, 0.999), (3.0, 0.5)]
+    us = [0.003, 0.21, 0.5, 0.77, 0.9991]
+    rows = [(t, p, u) for t, p in cases for u in us]
+    logits = base.expand(len(rows), vocab).contiguous()
+    got = run_sample(ops, logits, [r[0] for r in rows], [r[1] for r in rows], [r[2] for r in rows])
+    for (t, p, u), tok in zip(rows, got):
+        if t == 0.0:
+            assert tok == int(base.argmax())
+            continue
+        kept, weights = plain.softmax_sample_reference(base, t, p)
+        order = kept.argsort()
+        ids, w = kept[order], weights[order]
+        assert tok in set(ids.tolist()), f"T={t} top_p={p}: token {tok} is outside the nucleus of {len(ids)}"
+        cum = (w / w.sum()).cumsum(0)
+        j = int(torch.searchsorted(cum, torch.tensor(u, dtype=torch.float64), right=True))
+        near = {int(ids[min(max(j + d, 0), len(ids) - 1)]) for d in (-2, -1, 0, 1, 2)}  # 24-bit weights
+        assert tok in near, f"T={t} top_p={p} u={u}: token {tok}, the plain rule draws {int(ids[min(j, len(ids) - 1)])}"
+    # rows that all keep everything: the short form gives the same tokens
+    plain_rows = [(t, 1.0, u) for t in (0.5, 1.0, 0.0) for u in us]
+    args = ([r[0] for r in plain_rows], [r[1] for r in plain_rows], [r[2] for r in plain_rows])
+    wide = base.expand(len(plain_rows), vocab).contiguous()
+    assert run_sample(ops, wide, *args, nucleus=False) == run_sample(ops, wide, *args, nucleus=True)
+
+
+def test_sample_with_equal_weights_across_chunks_and_with_holes(ops):
+    """20,000 equal logits (five chunks, more equal weights than the threshold search
+    holds in LDS): top_p 0.35 keeps the 7,000 with the lowest indices, and the draw is
+    uniform over them.  -inf and NaN entries are never drawn."""
+    vocab = 20000
+    us = [i / 50 + 0.004 for i in range(50)]
+    got = run_sample(ops, torch.zeros(50, vocab), [1.0] * 50, [0.35] * 50, us)
+    assert all(abs(tok - int(u * 7000)) <= 1 for tok, u in zip(got, us)), got
+    holes = torch.randn(vocab)
+    holes[::3] = float("-inf")
+    holes[1::3] = float("nan")
+    got = run_sample(ops, holes.expand(50, vocab).contiguous(), [2.0] * 50, [0.95] * 50, us)
+    assert all(tok % 3 == 2 for tok in got)
+    got = run_sample(ops, holes.expand(50, vocab).contiguous(), [2.0] * 50, [1.0] * 50, us, nucleus=False)
+    assert all(tok % 3 == 2 for tok in got)
+    # nothing has any weight: the argmax's answer (index 0)
+    assert run_sample(ops, torch.full((2, 5000), float("-inf")), [1.0, 1.0], [0.9, 1.0], [0.3, 0.6]) == [0, 0]
+
+
+def test_sample_refuses_a_scratch_that_is_too_small(ops):
+    from shrike_amd.kernels import KernelError
+
+    logits = torch.zeros(2, 5000, device="cuda")
+    f = lambda x: torch.tensor(x, dtype=torch.float32, device="cuda")  # noqa: E731
+    with pytest.raises(KernelError, match="scratch"):
+        ops.sample(logits, torch.empty(2, dtype=torch.int32, device="cuda"), f([1.0, 1.0]), f([0.9, 0.9]),
+                   f([0.5, 0.5]), torch.empty(2 * 5000, device="cuda"))
 
 
 def test_sample_frequencies_follow_the_distribution(ops):
