@@ -111,14 +111,15 @@ def make_engine(cfg, spec, max_batch: int, seed: int, budget: int | None = None)
 
 
 def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int,
-               prompt_len: int = PROMPT_LEN) -> dict:
+               prompt_len: int = PROMPT_LEN, temperature: float = 0.0, top_p: float = 1.0) -> dict:
     """Prefill `batch` prompts of `prompt_len` tokens, then time `steps` decode steps."""
     import torch
 
     from shrike_amd import SamplingParams
 
     rng = random.Random(seed)
-    sampling = SamplingParams(max_new_tokens=batch + warmup + steps + 8, ignore_eos=True)
+    sampling = SamplingParams(max_new_tokens=batch + warmup + steps + 8, ignore_eos=True,
+                              temperature=temperature, top_p=top_p)
     for _ in range(batch):
         engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], sampling)
     while engine.scheduler.waiting or not all(r.prefill_done for r in engine.scheduler.running):
@@ -392,6 +393,13 @@ def main() -> int:
             far[b] = run_decode(engine, cfg, b, far_steps, args.warmup, args.seed + 100 + b, args.far_context)
             print(f"[bench] batch {b} at context {far[b]['context_start']:.0f}: {far[b]['tok_s']:.1f} tok/s, "
                   f"{far[b]['ms_per_step']:.3f} ms/step, {far[b]['gb_s']:.0f} GB/s", file=sys.stderr)
+    # the main batch once more with temperature and a nucleus instead of the argmax, a short run
+    sampled = None
+    if not args.no_points:
+        sampled = run_decode(engine, cfg, args.batch, min(args.steps, 200), args.warmup, args.seed + 200 + args.batch,
+                             args.context, temperature=0.8, top_p=0.95)
+        print(f"[bench] batch {args.batch}, temperature 0.8, top_p 0.95: {sampled['tok_s']:.1f} tok/s, "
+              f"{sampled['ms_per_step']:.3f} ms/step", file=sys.stderr)
     prefill = run_prefill(engine, cfg, args.seed)
     print(f"[bench] prefill: {prefill}", file=sys.stderr)
     # one batch left running for the per-kernel times
@@ -465,6 +473,8 @@ def main() -> int:
     line["points"][f"decode_b{args.batch}"] = round(main_run["tok_s"], 1)
     for b, r in far.items():
         line["points"][f"decode_b{b}_ctx4000"] = round(r["tok_s"], 1)
+    if sampled:
+        line["points"][f"decode_b{args.batch}_top_p"] = round(sampled["tok_s"], 1)
     if peaks:
         line["roofline"]["achievable"] = peaks["copy_gbs"]
         line["roofline"]["achievable_read"] = peaks["read_gbs"]
