@@ -48,6 +48,8 @@ class Sampler:
         self.device = device
         self.engine_seed = engine_seed
         self._scratch = None
+        self._staging = None  # two page-locked buffers for the rows' parameters, used by turns
+        self._params = None
 
     def request_seed(self, req) -> int:
         if req.sampling.seed is not None:
@@ -74,17 +76,35 @@ class Sampler:
         if all(r.sampling.temperature == 0.0 for r in reqs):
             ops.argmax(logits, out)
             return
-        params = torch.tensor(
+        params = self._upload(
             [[r.sampling.temperature for r in reqs],
              [r.sampling.top_p for r in reqs],
              [uniform(self.request_seed(r), r.num_generated) for r in reqs]],
-            dtype=torch.float32,
-        ).to(logits.device)
+            logits.device,
+        )
         need = ops.sample_scratch_floats(rows, vocab)
         if self._scratch is None or self._scratch.numel() < need:
             self._scratch = torch.empty(need, dtype=torch.float32, device=logits.device)
         nucleus = any(r.sampling.temperature > 0.0 and r.sampling.top_p < 1.0 for r in reqs)
         ops.sample(logits, out, params[0], params[1], params[2], self._scratch, nucleus=nucleus)
+
+    def _upload(self, rows_of_floats: list, device) -> torch.Tensor:
+        """float32 [3, R] on the device without a wait: through one of two page-locked
+        buffers by turns and a copy kernel in stream order (a copy from ordinary memory
+        would hold the host until the step before it has finished on the device)."""
+        n = len(rows_of_floats[0])
+        turn = self._turn = 1 - getattr(self, "_turn", 0)
+        if self._staging is None or self._staging[0][0].shape[1] < n:
+            width = max(64, 2 * n)
+            self._staging = [(torch.empty(3, width, dtype=torch.float32, pin_memory=True), torch.cuda.Event())
+                             for _ in range(2)]
+            self._params = torch.empty(3, width, dtype=torch.float32, device=device)
+        host, read = self._staging[turn]
+        read.synchronize()  # the copy that last read this buffer has run
+        host[:, :n] = torch.tensor(rows_of_floats, dtype=torch.float32)
+        ops.copy_words(host.view(torch.int32), self._params.view(torch.int32))
+        read.record()
+        return self._params[:, :n]
 
     def sample(self, logits: torch.Tensor, reqs: list) -> list[int]:
         """The tokens themselves: launch(), then the wait for the device."""
