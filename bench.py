@@ -54,6 +54,9 @@ SHAPE_7B = {
 # the other shapes of the Qwen2.5 family that the engine is sized for: what differs from 7B
 SHAPES = {
     "7b": {},
+    "0.5b": {"hidden_size": 896, "intermediate_size": 4864, "num_hidden_layers": 24,
+             "num_attention_heads": 14, "num_key_value_heads": 2, "head_dim": 64, "vocab_size": 151936,
+             "tie_word_embeddings": True},
     "14b": {"hidden_size": 5120, "intermediate_size": 13824, "num_hidden_layers": 48,
             "num_attention_heads": 40, "num_key_value_heads": 8, "rms_norm_eps": 1e-5},
     "32b": {"hidden_size": 5120, "intermediate_size": 27648, "num_hidden_layers": 64,
@@ -87,6 +90,43 @@ def prefill_flops(cfg, n: int) -> float:
     # causal attention: token p reads p + 1 keys, 2 products of head_dim each per head
     attn = 4.0 * cfg.head_dim * cfg.num_attention_heads * cfg.num_hidden_layers * n * (n + 1) / 2
     return linear + attn
+
+
+def run_offline(cfg, spec, requests: int, seed: int) -> dict:
+    """The reference's offline throughput run (bench/bench_engine.py:47-63, lengths as
+    bench/workload.py:15-22): `requests` short prompts, 32 to 256 new tokens each, greedy,
+    all handed to generate() at once, the engine with its defaults (512-token budget,
+    prefix caching on).  The prompts are random ids of 24 to 72 tokens instead of the
+    reference's sentences."""
+    import torch
+
+    from shrike_amd import SamplingParams
+    from shrike_amd.config import EngineConfig
+    from shrike_amd.engine.llm_engine import LLMEngine
+    from shrike_amd.engine.loading import random_model
+
+    model, runtime = random_model(spec, seed=seed, dtype="bfloat16")
+    rng = random.Random(seed)
+    prompts = [[rng.randrange(cfg.vocab_size) for _ in range(rng.randint(24, 72))] for _ in range(requests)]
+    sampling = [SamplingParams(max_new_tokens=rng.randint(32, 256), ignore_eos=True) for _ in range(requests)]
+    defaults = EngineConfig(dtype="bfloat16", seed=seed)
+    pages = requests * (-(-(72 + 256) // defaults.block_size) + 1)
+    engine = LLMEngine(None, EngineConfig(dtype="bfloat16", seed=seed, num_kv_blocks=pages), model=model,
+                       runtime=runtime)
+    engine.generate(prompts[:4], SamplingParams(max_new_tokens=4, ignore_eos=True), chat=False)  # first launches
+    torch.cuda.synchronize()
+    steps_before = engine.metrics()["steps"]
+    t0 = time.perf_counter()
+    outputs = engine.generate(prompts, sampling, chat=False)
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    tokens = sum(len(o) for o in outputs)
+    assert [len(o) for o in outputs] == [s.max_new_tokens for s in sampling]
+    m = engine.metrics()
+    return {"tokens": tokens, "seconds": round(seconds, 4), "tok_s": round(tokens / seconds, 1),
+            "steps": m["steps"] - steps_before, "preemptions": m["preemptions"],
+            "prefix_cache_hit_rate": m["prefix_cache_hit_rate"], "max_running": defaults.max_running,
+            "token_budget": defaults.max_tokens_per_step, "page_size": defaults.block_size}
 
 
 def make_engine(cfg, spec, max_batch: int, seed: int, budget: int | None = None):
@@ -330,10 +370,13 @@ def main() -> int:
     ap.add_argument("--no-peaks", action="store_true",
                     help="skip the measurement of this GPU's copy bandwidth and product rate")
     ap.add_argument("--shape", choices=sorted(SHAPES), default="7b",
-                    help="layer sizes: Qwen2.5-7B (the default and the reported figure), 14B or 32B")
+                    help="layer sizes: Qwen2.5-7B (the default and the reported figure), 0.5B, 14B or 32B")
     ap.add_argument("--mixed", type=int, default=0, metavar="DECODES",
                     help="instead: time steps of DECODES single tokens plus a portion of a 2,048-token "
                          "prompt under a 512-token budget (prints its own JSON line)")
+    ap.add_argument("--offline", type=int, default=0, metavar="REQUESTS",
+                    help="instead: the reference's offline throughput run, REQUESTS short prompts with 32 to "
+                         "256 new tokens each through generate() (prints its own JSON line)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -362,6 +405,18 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
+    if args.offline:
+        offline = run_offline(cfg, spec, args.offline, args.seed)
+        print(json.dumps({
+            "metric": f"generated tok/s of {args.offline} requests with 32 to 256 new tokens each through "
+                      f"generate() (Qwen2.5-{args.shape.upper()} shape)",
+            "value": offline["tok_s"], "unit": "tok/s", "n_gpus": 1, "higher_is_better": True, "dtype": "bf16",
+            "data": "synthetic: random weights N(0, 0.02), prompts of 24 to 72 random ids",
+            "config": {"model": f"Qwen2.5-{args.shape.upper()} shape (Qwen2ForCausalLM)",
+                       "layers": cfg.num_hidden_layers, "layers_of_config": layers_of_config,
+                       "requests": args.offline, "sampling": "greedy"},
+            **offline}))
+        return 0
     if args.mixed:
         engine = make_engine(cfg, spec, args.mixed + 1, args.seed, budget=512)
         mixed = run_mixed(engine, cfg, args.mixed, 512, args.seed)
