@@ -1323,6 +1323,11 @@ extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   } else {
     split = 2048 / mblocks, most = ktiles / 28;
     if (split > 8) split = 8;
+    // a small matrix (896 x 896 has 56 blocks: 14 workgroups) is a matter of how long one
+    // wavefront walks, not of what its shares cost: shares down to two stages of four tiles
+    // (with 64 tokens 896 x 896 takes 6 us in 3 shares against 10.5 whole)
+    const int with_most = split < most ? split : most;
+    if (mblocks * (with_most > 1 ? with_most : 1) < 512) most = ktiles / 8;
   }
   if (split > most) split = most;
   return split > 1 ? split : 1;
