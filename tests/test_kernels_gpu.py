@@ -439,6 +439,11 @@ def test_sample_refuses_a_scratch_that_is_too_small(ops):
     with pytest.raises(KernelError, match="scratch"):
         ops.sample(logits, torch.empty(2, dtype=torch.int32, device="cuda"), f([1.0, 1.0]), f([0.9, 0.9]),
                    f([0.5, 0.5]), torch.empty(2 * 5000, device="cuda"))
+    # and a row of more than 1024 chunks of 4096
+    wide = torch.zeros(1, 1024 * 4096 + 1, device="cuda")
+    with pytest.raises(KernelError, match="beyond"):
+        ops.sample(wide, torch.empty(1, dtype=torch.int32, device="cuda"), f([1.0]), f([0.9]), f([0.5]),
+                   torch.empty(ops.sample_scratch_floats(1, wide.shape[1]), device="cuda"))
 
 
 def test_sample_frequencies_follow_the_distribution(ops):
