@@ -34,34 +34,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # Qwen2.5-7B shape
-SHAPE_7B = {
-    "architectures": ["Qwen2ForCausalLM"],
-    "hidden_size": 3584,
-    "intermediate_size": 18944,
-    "num_hidden_layers": 28,
-    "num_attention_heads": 28,
-    "num_key_value_heads": 4,
-    "head_dim": 128,
-    "vocab_size": 152064,
-    "rope_theta": 1000000.0,
-    "rms_norm_eps": 1e-6,
-    "tie_word_embeddings": False,
-    "attention_bias": True,
-    "max_position_embeddings": 32768,
-    "eos_token_id": 151645,
-    "torch_dtype": "bfloat16",
-}
-# the other shapes of the Qwen2.5 family that the engine is sized for: what differs from 7B
-SHAPES = {
-    "7b": {},
-    "0.5b": {"hidden_size": 896, "intermediate_size": 4864, "num_hidden_layers": 24,
-             "num_attention_heads": 14, "num_key_value_heads": 2, "head_dim": 64, "vocab_size": 151936,
-             "tie_word_embeddings": True},
-    "14b": {"hidden_size": 5120, "intermediate_size": 13824, "num_hidden_layers": 48,
-            "num_attention_heads": 40, "num_key_value_heads": 8, "rms_norm_eps": 1e-5},
-    "32b": {"hidden_size": 5120, "intermediate_size": 27648, "num_hidden_layers": 64,
-            "num_attention_heads": 40, "num_key_value_heads": 8, "rms_norm_eps": 1e-5},
-}
+# layer sizes: the config.json files that the package ships as data
+def _shape(name: str) -> dict:
+    from shrike_amd.config.presets import load_preset
+
+    return load_preset(f"qwen2.5-{name}")
+
+
+SHAPE_NAMES = ("0.5b", "7b", "14b", "32b")
 PROMPT_LEN = 2048
 CONTEXT_END = 4096
 PAGE_SIZE = 16
@@ -357,7 +337,7 @@ def main() -> int:
                     help="timed decode steps; 1900 after 2048-token prompts reach context 4,000")
     ap.add_argument("--warmup", type=int, default=4)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=SHAPE_7B["num_hidden_layers"],
+    ap.add_argument("--layers", type=int, default=None,
                     help="run fewer layers than the configuration has (both numbers are reported)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--context", type=int, default=PROMPT_LEN, metavar="N",
@@ -369,7 +349,7 @@ def main() -> int:
                     help="context of the extra points decode_b*_ctx4000 (0: leave them out)")
     ap.add_argument("--no-peaks", action="store_true",
                     help="skip the measurement of this GPU's copy bandwidth and product rate")
-    ap.add_argument("--shape", choices=sorted(SHAPES), default="7b",
+    ap.add_argument("--shape", choices=SHAPE_NAMES, default="7b",
                     help="layer sizes: Qwen2.5-7B (the default and the reported figure), 0.5B, 14B or 32B")
     ap.add_argument("--mixed", type=int, default=0, metavar="DECODES",
                     help="instead: time steps of DECODES single tokens plus a portion of a 2,048-token "
@@ -399,9 +379,9 @@ def main() -> int:
     import shrike_amd.models  # noqa: F401
     from shrike_amd.models.qwen2 import Qwen2Config, build_spec
 
-    raw = dict(SHAPE_7B, **SHAPES[args.shape])
+    raw = _shape(args.shape)
     layers_of_config = raw["num_hidden_layers"]
-    if args.layers != SHAPE_7B["num_hidden_layers"] or args.shape == "7b":
+    if args.layers is not None:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)

@@ -23,8 +23,9 @@ def parse_args(argv=None) -> argparse.Namespace:
     ap.add_argument("prompt", nargs="?", default=None, help="text prompt (needs tokenizer.json)")
     ap.add_argument("--model", default=DEFAULT_MODEL_DIR)
     ap.add_argument("--random-config", default=None, metavar="CONFIG_JSON",
-                    help="instead of --model: a config.json (or a folder with one) whose architecture "
-                         "is built with random weights drawn on the device from --seed")
+                    help="instead of --model: a config.json (or a folder with one, or the name of a preset: "
+                         "qwen2.5-0.5b, -7b, -14b, -32b) whose architecture is built with random weights "
+                         "drawn on the device from --seed")
     ap.add_argument("--prompt-ids", default=None, help="comma-separated token ids")
     ap.add_argument("--prompt-len", type=int, default=None, help="that many random token ids")
     ap.add_argument("--max-tokens", type=int, default=128)
@@ -65,14 +66,19 @@ def main(argv=None) -> int:
         from .config import EngineConfig, architecture_name, canonical_dtype, get_architecture
         from .engine.loading import random_model
 
+        from .config.presets import load_preset, preset_names
+
         path = args.random_config
         if os.path.isdir(path):
             path = os.path.join(path, "config.json")
         try:
-            with open(path) as f:
-                raw = json.load(f)
+            if not os.path.exists(path) and path.lower() in preset_names():
+                raw = load_preset(path)
+            else:
+                with open(path) as f:
+                    raw = json.load(f)
         except (OSError, ValueError) as e:
-            print(f"[error] --random-config {path}: {e}", file=sys.stderr)
+            print(f"[error] --random-config {path}: {e} (presets: {', '.join(preset_names())})", file=sys.stderr)
             return 2
         arch = get_architecture(architecture_name(raw))
         spec = arch.build_spec(arch.config_cls.from_dict(raw))
