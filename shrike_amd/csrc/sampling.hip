@@ -374,7 +374,6 @@ __global__ void __launch_bounds__(kThresholdThreads)
   __shared__ u64 held[kBoundaryInLds];
   __shared__ uint32_t first[kMaxChunks + 1];  // where a chunk's collected weights start
   __shared__ u64 digit_mass[2][256];
-  __shared__ u64 passed;  // mass of the digits above the chosen one
   __shared__ float fscratch[16];
   __shared__ u64 uscratch[17];
   const int row = blockIdx.x;
@@ -425,12 +424,15 @@ __global__ void __launch_bounds__(kThresholdThreads)
 
   // tau's high bits are the class's; the open ones are found eight at a time: among the
   // weights that share the bits found so far, the mass by the next eight bits, and from
-  // the top the digit at which the upper mass reaches `need`
+  // the top the digit at which the upper mass reaches `need`.  A weight is a float's 24
+  // bits shifted: below those every weight has zeros, which need no search.
   int open_bits;
   u64 found = class_base(st.boundary, &open_bits) >> open_bits;  // the bits known so far
   u64 above = st.above;                                          // mass of the weights above them
-  for (int phase = 0; open_bits > 0; ++phase) {
-    const int width = open_bits < 8 ? open_bits : 8, shift = open_bits - width;
+  const int zero_bits = open_bits > 20 ? open_bits - 20 : 0;     // (4 bits are the class's, 20 more may differ)
+  const int lane = threadIdx.x & (kWave - 1);
+  for (int phase = 0; open_bits > zero_bits; ++phase) {
+    const int width = open_bits - zero_bits < 8 ? open_bits - zero_bits : 8, shift = open_bits - width;
     u64* mass = digit_mass[phase & 1];
     if (threadIdx.x < 256) mass[threadIdx.x] = 0;
     __syncthreads();
@@ -438,19 +440,33 @@ __global__ void __launch_bounds__(kThresholdThreads)
       if ((q >> open_bits) == found) atomicAdd(&mass[(q >> shift) & ((1u << width) - 1)], q);
     });
     __syncthreads();
-    // thread t < 256 takes digit 255 - t: the prefix sums in thread order are the masses above a digit
-    const int d = 255 - static_cast<int>(threadIdx.x);
-    const u64 mine = d >= 0 ? mass[d] : 0;
-    u64 heavier, all;
-    block_scan_u64(mine, uscratch, &heavier, &all);
-    const bool reached = d >= 0 && above + heavier + mine >= st.need;
-    const int digit = static_cast<int>(block_max(reached ? static_cast<float>(d) : 0.f, fscratch));
-    if (d == digit) passed = heavier;
-    __syncthreads();
-    above += passed;
+    // Every wavefront finds the digit by itself, from the same 256 sums: lane l takes the
+    // digits 255 - 4 l down to 252 - 4 l, a prefix sum over the lanes gives the mass above
+    // them, and the first lane (highest digits) in which the upper mass reaches `need` tells.
+    u64 own[4], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) own[i] = mass[255 - (4 * lane + i)], sum += own[i];
+    u64 upto = sum;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const u64 o = __shfl_up(upto, off, kWave);
+      if (lane >= off) upto += o;
+    }
+    u64 run = upto - sum, run_at_hit = 0;
+    int hit = -1;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (hit < 0 && above + run + own[i] >= st.need) hit = i, run_at_hit = run;
+      run += own[i];
+    }
+    const unsigned long long reached = __ballot(hit >= 0);
+    const int teller = reached ? __ffsll(reached) - 1 : kWave - 1;  // (some lane always reaches it)
+    const int digit = __shfl(hit >= 0 ? 255 - (4 * lane + hit) : 0, teller, kWave);
+    above += __shfl(hit >= 0 ? run_at_hit : run, teller, kWave);
     found = (found << width) | static_cast<u64>(digit);
     open_bits = shift;
   }
+  found <<= open_bits;  // the bits that are zero in every weight
   const u64 tau = found;  // `above` is now the mass of all weights above tau
   u64 equal = 0;
   for_all([&](u64 q) { equal += q == tau; });
