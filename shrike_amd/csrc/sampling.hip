@@ -90,7 +90,7 @@ __global__ void __launch_bounds__(kArgmaxThreads)
 
 // ------------------------------------------------------ temperature / top-p
 // A row of 152,064 logits is too long for one workgroup to walk a few dozen
-// times (the first form of this did: 0.3 to 1.8 ms a step), so a row is cut into
+// times (that takes 0.3 to 1.8 ms a step, with the batch), so a row is cut into
 // chunks of 4096 like the wide argmax, every pass over the logits is a launch of
 // chunks x rows workgroups, and short single-workgroup kernels between them
 // decide.  Weights are integers, floor(exp((x - max) / T) * 2^40): sums of
