@@ -431,6 +431,49 @@ def test_sample_with_equal_weights_across_chunks_and_with_holes(ops):
     assert run_sample(ops, torch.full((2, 5000), float("-inf")), [1.0, 1.0], [0.9, 1.0], [0.3, 0.6]) == [0, 0]
 
 
+def test_sample_random_rows_follow_the_plain_rule(ops):
+    """Rows of many widths (one chunk, a chunk's edge, many chunks), spreads (flat to
+    peaked), rounded logits with many equal weights, holes of -inf, temperatures and
+    nuclei: the token lies in the plain rule's kept set and near the inverse of its
+    cumulative kept weight in index order.  Entries whose membership hangs on less than
+    1e-5 of the mass may go either way (the engine's weights have 24 bits)."""
+    import random
+
+    for seed in range(120):
+        rng = random.Random(seed)
+        torch.manual_seed(seed)
+        vocab = rng.choice([2, 3, 17, 1000, 4095, 4096, 4097, 8191, 20000, 50000, 152064])
+        rows = rng.choice([1, 2, 5])
+        logits = torch.randn(rows, vocab) * rng.choice([0.0, 0.1, 1.0, 5.0, 20.0])
+        if rng.random() < 0.3:
+            logits = (logits * 2).round() / 2
+        if rng.random() < 0.2 and vocab > 10:
+            logits[:, rng.randrange(vocab)] = float("-inf")
+        temps = [rng.choice([0.0, 0.05, 0.3, 0.7, 1.0, 2.0, 5.0]) for _ in range(rows)]
+        tops = [rng.choice([0.01, 0.1, 0.5, 0.9, 0.95, 0.999, 1.0]) for _ in range(rows)]
+        us = [rng.random() for _ in range(rows)]
+        nucleus = any(t > 0 and p < 1 for t, p in zip(temps, tops)) or rng.random() < 0.5
+        got = run_sample(ops, logits, temps, tops, us, nucleus=nucleus)
+        for r, tok in enumerate(got):
+            t, p, u = (float(torch.tensor(x, dtype=torch.float32)) for x in (temps[r], tops[r], us[r]))
+            case = f"seed {seed} row {r}: vocab {vocab} T {t} top_p {p} u {u}: token {tok}"
+            if t == 0.0:
+                assert tok == int(logits[r].argmax()), case
+                continue
+            probs = torch.softmax(logits[r].double() / t, -1)
+            sp, si = probs.sort(descending=True, stable=True)
+            before = sp.cumsum(0) - sp
+            keep, slack = before < p, (before - p).abs() < 1e-5
+            either = set(si[slack].tolist())
+            assert tok in set(si[keep].tolist()) | either, case + " is outside the nucleus"
+            ids = si[keep].sort().values
+            cum = probs[ids].cumsum(0) / probs[ids].sum()
+            lo = int(torch.searchsorted(cum, torch.tensor(max(u - 1e-4, 0.0), dtype=torch.float64), right=True))
+            hi = int(torch.searchsorted(cum, torch.tensor(min(u + 1e-4, 1.0), dtype=torch.float64), right=True))
+            near = set(ids[max(lo - 1, 0): min(hi + 2, len(ids))].tolist()) | either
+            assert tok in near, case + f", the plain rule draws {int(ids[min(lo, len(ids) - 1)])}"
+
+
 def test_sample_refuses_a_scratch_that_is_too_small(ops):
     from shrike_amd.kernels import KernelError
 
