@@ -504,12 +504,16 @@ __global__ void __launch_bounds__(kChunkThreads)
   __shared__ u64 found[3];  // the chunk of the draw, the kept mass and the equal weights before it
   const int row = blockIdx.x;
   const size_t rc0 = static_cast<size_t>(row) * chunks;
-  // the argmax: chunks are in index order, so the first maximum among them has the lowest index
-  const MaxIdx best = block_argmax(s.best_value + rc0, chunks, mscratch);
-  const int greedy = s.best_index[rc0 + best.i];
+  // the argmax (only where it is the answer): chunks are in index order, so the first
+  // maximum among them has the lowest index
+  const auto greedy = [&]() {
+    const MaxIdx best = block_argmax(s.best_value + rc0, chunks, mscratch);
+    return s.best_index[rc0 + best.i];
+  };
   const float temp = temperature[row];
   if (!(temp > 0.f)) {
-    if (threadIdx.x == 0) out[row] = greedy;
+    const int token = greedy();
+    if (threadIdx.x == 0) out[row] = token;
     return;
   }
   u64 tau = 0;
@@ -544,7 +548,8 @@ __global__ void __launch_bounds__(kChunkThreads)
   u64 run, kept;
   block_scan_u64(mass_sum, uscratch, &run, &kept);
   if (kept == 0) {  // nothing has any weight (a row of NaN): the argmax's answer
-    if (threadIdx.x == 0) out[row] = greedy;
+    const int token = greedy();
+    if (threadIdx.x == 0) out[row] = token;
     return;
   }
   u64 target = static_cast<u64>(static_cast<double>(uniforms[row]) * static_cast<double>(kept));
@@ -592,7 +597,7 @@ __global__ void __launch_bounds__(kChunkThreads)
   // exactly one thread's kept weights span the target
   if (my_mass > 0 && mass_before <= target && target < mass_before + my_mass) {
     u64 passed = mass_before;
-    int token = greedy;
+    int token = begin;  // (always replaced: the thread's kept mass spans the target)
     bool done = false;
 #pragma unroll
     for (int k = 0; k < kPerThread; ++k) {  // the first kept entry at which the running mass passes the target
