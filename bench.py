@@ -263,6 +263,9 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
         return timed
 
     runner = engine.runner
+    # no step may be in flight or planned from before: the next ones are to run kernel by kernel
+    overlap, engine.config.overlap_steps = engine.config.overlap_steps, False
+    engine.step()  # takes in the step that was launched ahead, if one was, and launches none
     graphs, runner.use_graphs = runner.use_graphs, False
     engine._planned = None
     try:
@@ -281,6 +284,7 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
         for n, fn in saved.items():
             setattr(ops, n, fn)
         runner.use_graphs = graphs
+        engine.config.overlap_steps = overlap
         engine._planned = None
     total: dict[str, float] = {}
     for label, a, b in spans:
@@ -492,7 +496,7 @@ def main() -> int:
             "page_size": PAGE_SIZE,
             "parallelism": "single GPU",
             "sampling": "greedy",
-            "hip_graphs": True,
+            "hip_graphs": bool(engine.config.graphs and engine.runner.use_graphs),
         },
         "prefill": prefill,
         "roofline": {

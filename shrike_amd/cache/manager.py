@@ -179,7 +179,10 @@ class CacheManager:
         slot = self.slots.take()
         for g in self.state_groups:
             if g.tensor is not None:
-                g.tensor[:, slot].zero_()
+                from ..kernels import ops
+
+                for layer in range(g.tensor.shape[0]):
+                    ops.zero_(g.tensor[layer, slot])
         return SequenceCache(
             tables=[[] for _ in self.groups], state_slot=slot, _trimmed=[0] * len(self.groups)
         )

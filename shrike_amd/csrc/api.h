@@ -21,6 +21,21 @@ int shk_version(void);
 int shk_copy_words(const int32_t* src, int32_t* dst, int n, const int32_t* patch, int patch_at,
                    int patch_n, void* stream);
 
+// dst[r, :] = src[index[r], :] for r < rows: rows of `width` 32-bit words, src rows
+// `ld` words apart; the caller promises 0 <= index[r] < src_rows.  index may be
+// page-locked host memory.
+int shk_gather_rows(const int32_t* src, long long ld, int src_rows, const int32_t* index, int32_t* dst,
+                    int rows, int width, void* stream);
+
+// Reads `bytes` bytes from p (16-byte aligned) with `workgroups` workgroups of 512
+// threads and keeps nothing: a kernel that needs them next finds them in the caches
+// between the compute units and memory.  sink may be null.
+int shk_touch(const void* p, long long bytes, int workgroups, int32_t* sink, void* stream);
+
+// Zeroes `bytes` bytes from dst, which must be 4-byte aligned (a fill kernel:
+// it may be recorded into a HIP graph).
+int shk_zero_bytes(void* dst, long long bytes, void* stream);
+
 // out[i, :] = float(table[ids[i], :]); ids must lie in [0, vocab).
 int shk_embed(const void* table, int dtype, const int32_t* ids, float* out, int n, int hidden,
               int vocab, void* stream);

@@ -1197,10 +1197,7 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
   // second) and at least 128 tokens (with 64 it measured 3 % slower).
   if constexpr (GM * GN >= 8 && GN * WN >= 8 &&
                 3 * (GM * WM + GN * WN) * KS * kWave * 16 <= 160 * 1024) {
-    // (SHK_NO_LDS_LOADS=1 in the environment keeps to the kernel that stages through
-    // registers: for comparing the two)
-    static const bool direct = getenv("SHK_NO_LDS_LOADS") == nullptr;
-    if (direct && vec && kt % KS == 0) {
+    if (vec && kt % KS == 0) {
       if (gated)
         gemm_big_lds_kernel<GM, GN, WM, WN, KS, true><<<grid, GM * GN * kWave, 0, s>>>(
             ap, lda, n, k, wp, kt, m, bias, out, ldo, of, accumulate, ksplit, tiles_x, tiles_y, by_die);

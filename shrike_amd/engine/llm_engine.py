@@ -80,6 +80,7 @@ class LLMEngine:
         # (batch, logits) of a decode step that is already running on the device: it was
         # launched, fed with the last step's tokens on the device, before the host read them
         self._inflight = None
+        self._row_list = self._row_list_read = None  # page-locked row indices for _rows_of
 
     # reference name for the cache manager
     @property
@@ -91,22 +92,21 @@ class LLMEngine:
             token_ids = _encode(self.tokenizer, self.model_dir, prompt, chat)
         else:
             token_ids = [int(t) for t in prompt]
-        if not token_ids:
-            raise ValueError(
-                "empty prompt: a request must have at least one token "
-                "(the prompt tokenized to zero tokens)"
-            )
+        if len(token_ids) == 0:
+            raise ValueError("a request with an empty prompt cannot be served: there is no token "
+                             "to compute a next one from")
         vocab = self.model.spec.vocab_size
         if min(token_ids) < 0 or max(token_ids) >= vocab:
             raise ValueError(f"prompt token ids must lie in [0, {vocab})")
-        bs = self.cache.page_size
-        worst = -(-(len(token_ids) + sampling.max_new_tokens) // bs)
-        if worst > self.cache.num_pages:
+        page = self.cache.page_size
+        longest = len(token_ids) + sampling.max_new_tokens
+        pages_at_most = -(-longest // page)
+        if pages_at_most > self.cache.num_pages:
             raise ValueError(
-                f"request needs up to {worst} KV blocks ({len(token_ids)} prompt + "
-                f"{sampling.max_new_tokens} generated tokens, block_size={bs}) but the pool has "
-                f"only {self.cache.num_pages}; it could never be scheduled - shorten the prompt, "
-                "lower max_new_tokens, or raise gpu_mem_util / num_kv_blocks"
+                f"this request could never be scheduled: {len(token_ids)} prompt tokens and up to "
+                f"{sampling.max_new_tokens} new ones fill {pages_at_most} pages of {page} tokens, and "
+                f"the whole pool is {self.cache.num_pages} pages.  A shorter prompt, a smaller "
+                "max_new_tokens or a larger pool (num_kv_blocks, gpu_mem_util) would let it in"
             )
         req = Request(token_ids=token_ids, sampling=sampling, req_id=self._next_req_id)
         self._next_req_id += 1
@@ -131,8 +131,7 @@ class LLMEngine:
                     if req.status is Status.RUNNING and self.requests.get(req.req_id) is req]
             if live:
                 batch = [launched[i] for i in live]
-                logits = all_logits if len(live) == len(launched) else all_logits[
-                    torch.tensor(live, dtype=torch.long, device=all_logits.device)]
+                logits = all_logits if len(live) == len(launched) else self._rows_of(all_logits, live)
                 sampled = [req for req, _ in batch]
         if batch is None:
             planned, self._planned = self._planned, None
@@ -193,18 +192,38 @@ class LLMEngine:
         self.stats.steps += 1
         return outputs
 
+    def _rows_of(self, logits: torch.Tensor, rows: list[int]) -> torch.Tensor:
+        """The given rows of `logits`, gathered by a kernel whose row list lies in
+        page-locked memory (no copy of it to the device, no library indexing)."""
+        from ..kernels import ops
+
+        if self._row_list is None or self._row_list.numel() < len(rows):
+            self._row_list = torch.empty(max(256, len(rows)), dtype=torch.int32, pin_memory=True)
+            self._row_list_read = torch.cuda.Event()
+        else:
+            self._row_list_read.synchronize()  # the last gather has read the list
+        index = self._row_list[: len(rows)]
+        index.numpy()[:] = rows
+        out = self.runner.workspace.get("live_logits", (len(rows), logits.shape[1]), logits.dtype)
+        ops.gather_rows(logits, index, out)
+        self._row_list_read.record()
+        return out
+
     def generate(self, prompts, sampling, chat: bool = True) -> list[list[int]]:
-        """Generated token ids per prompt (the end-of-sequence token included when hit)."""
-        if isinstance(sampling, SamplingParams):
-            sampling = [sampling] * len(prompts)
-        if len(sampling) != len(prompts):
+        """Runs the prompts to their ends; the tokens generated for each, in the
+        order of `prompts` (an end-of-sequence token that ended one is its last)."""
+        prompts = list(prompts)
+        per_prompt = [sampling] * len(prompts) if isinstance(sampling, SamplingParams) else list(sampling)
+        if len(per_prompt) != len(prompts):
             raise ValueError("one SamplingParams per prompt, or one for all")
-        id_map = {self.add_request(p, s, chat): i for i, (p, s) in enumerate(zip(prompts, sampling))}
-        results: list[list[int]] = [[] for _ in prompts]
-        while self.has_work:
+        generated: dict[int, list[int]] = {}
+        for prompt, params in zip(prompts, per_prompt):
+            generated[self.add_request(prompt, params, chat)] = []
+        while self.scheduler.has_work:
             for out in self.step():
-                results[id_map[out.req_id]].append(out.token_id)
-        return results
+                if out.req_id in generated:  # a request added by someone else runs along unrecorded
+                    generated[out.req_id].append(out.token_id)
+        return list(generated.values())
 
     def abort(self, req_id: int) -> None:
         req = self.requests.pop(req_id, None)
@@ -238,6 +257,8 @@ def workspace_reserve(model, runtime, cfg: EngineConfig) -> int:
     of its own, each half the next one's size, so the largest counts twice."""
     from .runner import GRAPH_BATCH_BUCKETS, Workspace
 
+    from ..kernels import ops
+
     pages = -(-cfg.max_tokens_per_step // cfg.block_size) + 1
     cache = CacheManager(model.cache_specs(), cfg.block_size, pages, max_slots=2,
                          enable_prefix_caching=False)
@@ -251,8 +272,16 @@ def workspace_reserve(model, runtime, cfg: EngineConfig) -> int:
         runner.dry_run(singles, portion)
         sizes.append(runner.workspace.nbytes())
     torch.cuda.synchronize(runtime.device)
-    slack = 64 << 20  # graph objects, pinned staging, the sampler's scratch
-    return 2 * sizes[0] + sizes[1] + slack
+    # What the probe allocated goes back to the device, not only to torch's own pool of
+    # freed blocks: the caller reads the free memory next, and would otherwise count the
+    # probe's buffers twice, once as memory that is gone and once in this reserve.
+    del runner, cache
+    torch.cuda.empty_cache()
+    # the sampler's scratch for the largest batch that can want a token in one step
+    sampler = 4 * ops.sample_scratch_floats(min(cfg.max_running, cfg.max_tokens_per_step),
+                                            model.spec.vocab_size)
+    slack = 64 << 20  # graph objects, page-locked staging
+    return 2 * sizes[0] + sizes[1] + sampler + slack
 
 
 class LLM:

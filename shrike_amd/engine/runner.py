@@ -299,11 +299,14 @@ class ModelRunner:
                 # before the capture starts.  Recording executes nothing, so this
                 # run's logits are the step's result and the graph is not replayed
                 # now: a part that advances a state of its own must see each step once.
-                eager_logits = self.model.forward(g.ctx, self.layer_caches).clone()
+                eager_logits = self.model.forward(g.ctx, self.layer_caches)
                 torch.cuda.synchronize(self.runtime.device)
                 graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(graph):
                     g.logits = self.model.forward(g.ctx, self.layer_caches)
+                # The recording wrote nothing: eager_logits, be it the workspace buffer
+                # that the recorded run names too or a tensor that a part allocated for
+                # itself, still holds what the kernel-by-kernel run put there.
                 g.graph = graph
                 self._graphs[key] = g
                 self.graph_captures += 1

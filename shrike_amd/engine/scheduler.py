@@ -39,11 +39,12 @@ class Scheduler:
         self.num_preemptions = 0
 
     def add(self, req: Request) -> None:
+        """A new request queues behind those that wait already."""
         self.waiting.append(req)
 
     @property
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return len(self.running) + len(self.waiting) > 0
 
     def _release(self, req: Request) -> None:
         if req.cache is not None:
@@ -51,15 +52,15 @@ class Scheduler:
             req.cache = None
         req.hashed_pages, req.last_hash = 0, None
 
-    def _preempt_for(self, req: Request) -> bool:
-        """Preempt the newest running request; False if that was `req` itself."""
-        victim = self.running.pop()
+    def _preempt_newest(self) -> Request:
+        """The request admitted last loses its pages and its slot and goes to the
+        head of the waiting queue, to start over from its first token."""
+        newest = self.running.pop()
+        self._release(newest)
+        newest.status, newest.num_computed_tokens = Status.WAITING, 0
+        self.waiting.appendleft(newest)
         self.num_preemptions += 1
-        self._release(victim)
-        victim.num_computed_tokens = 0
-        victim.status = Status.WAITING
-        self.waiting.appendleft(victim)
-        return victim is not req
+        return newest
 
     def schedule(self) -> list[tuple[Request, int]]:
         singles: list[tuple[Request, int]] = []
@@ -74,10 +75,9 @@ class Scheduler:
             n_new = min(req.num_tokens - req.num_computed_tokens, budget)
             if n_new <= 0:
                 continue
-            while not self.cache.can_append(req.cache, req.num_computed_tokens, n_new):
-                if not self._preempt_for(req):
-                    n_new = 0
-                    break
+            while n_new and not self.cache.can_append(req.cache, req.num_computed_tokens, n_new):
+                if self._preempt_newest() is req:
+                    n_new = 0  # it was the newest itself: it sits this step out
             if n_new == 0:
                 continue
             self.cache.append(req.cache, req.num_computed_tokens, n_new)
@@ -146,10 +146,11 @@ class Scheduler:
             self.cache.trim(req.cache, req.num_computed_tokens)
 
     def finish(self, req: Request, reason: str) -> None:
-        req.status = Status.FINISHED
-        req.finish_reason = reason
+        """A running request is done: it leaves the running list and everything
+        it holds goes back to the cache manager."""
         self.running.remove(req)
         self._release(req)
+        req.status, req.finish_reason = Status.FINISHED, reason
 
     def abort(self, req: Request) -> None:
         """Drop a request wherever it is (command line interrupt)."""

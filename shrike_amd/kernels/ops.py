@@ -78,6 +78,38 @@ def copy_words(src: torch.Tensor, dst: torch.Tensor, patch: torch.Tensor | None 
                                 None if patch is None else _words(patch, "patch"), patch_at, patch_n, _stream()))
 
 
+def gather_rows(src: torch.Tensor, index: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst[r] = src[index[r]] for 2-d tensors of a 4-byte dtype (src rows may be
+    strided); index int32, on the device or page-locked, every entry below src's
+    row count (the caller's promise: nothing on the device checks it)."""
+    _rows(src, "gather_rows src")
+    if (dst.dim() != 2 or not dst.is_contiguous() or dst.dtype != src.dtype or src.element_size() != 4
+            or dst.shape[1] != src.shape[1] or index.numel() != dst.shape[0]):
+        raise KernelError("gather_rows: dst must be contiguous [len(index), width] of src's 4-byte dtype")
+    check(load().shk_gather_rows(_dev(src, "src"), src.stride(0), src.shape[0], _words(index, "index"),
+                                 _dev(dst, "dst"), dst.shape[0], dst.shape[1], _stream()))
+
+
+def touch(t: torch.Tensor, workgroups: int = 256, nbytes: int | None = None, offset: int = 0) -> None:
+    """Reads `nbytes` bytes of a contiguous device tensor from byte `offset` on (all of
+    it by default) and keeps nothing: the next kernel that needs them finds them in
+    the caches on the way to memory."""
+    if not t.is_contiguous():
+        raise KernelError("touch: expected a contiguous tensor")
+    total = t.numel() * t.element_size()
+    nbytes = total - offset if nbytes is None else nbytes
+    if offset < 0 or offset % 16 or nbytes < 0 or offset + nbytes > total:
+        raise KernelError("touch: the range does not lie within the tensor (offset in steps of 16 bytes)")
+    check(load().shk_touch(_dev(t, "t") + offset, nbytes, workgroups, None, _stream()))
+
+
+def zero_(t: torch.Tensor) -> None:
+    """Fills a contiguous device tensor with zero bytes by a kernel of the library."""
+    if not t.is_contiguous():
+        raise KernelError("zero_: expected a contiguous tensor")
+    check(load().shk_zero_bytes(_dev(t, "t"), t.numel() * t.element_size(), _stream()))
+
+
 def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
     """out[i] = float(table[ids[i]]); ids int32 [n], out float32 [n, hidden]."""
     n, hidden = out.shape

@@ -11,15 +11,23 @@ from ..kernels import ops
 from .base import Mixer, PagedKVSpec, ParamSpec, build_part, register_mixer
 
 QUERY_TILE = 16  # queries per tile of the MFMA kernels for prompt portions
-COMPUTE_UNITS = 256
+COMPUTE_UNITS = 256  # of an MI355X; compute_units() asks the device that is there
 KEYS_PER_WORKGROUP = 256  # a decode workgroup's four wavefronts want at least this many keys
 MAX_KEY_SPLITS = 64
 # decode attention fetches keys and values with non-temporal loads from this many bytes
 # of them per launch on (counted with the batch and the context rounded up to powers of two)
 STREAMING_FROM_BYTES = 96 << 20
-# prompt portions take workgroups of 8 wavefronts instead of 16 while no more than this many
-# of them are launched: two fit on a compute unit, so all of them run at once
-SMALL_WORKGROUPS_AT_ONCE = 2 * COMPUTE_UNITS
+_UNITS: int | None = None
+
+
+def compute_units() -> int:
+    """Compute units of the GPU the process runs on (read once; COMPUTE_UNITS where no
+    GPU is visible, so that launch plans can be computed and tested without one)."""
+    global _UNITS
+    if _UNITS is None:
+        _UNITS = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
+                  if torch.cuda.is_available() else COMPUTE_UNITS)
+    return _UNITS
 
 
 def _pow2(n: int, floor: int = 1) -> int:
@@ -35,7 +43,7 @@ def decode_splits(num_seqs: int, kv_heads: int, max_ctx: int) -> int:
     for its four wavefronts.  Both inputs are rounded up to powers of two first,
     so a step gives the same result whether it runs kernel by kernel or as a
     graph captured for a padded batch."""
-    want = -(-COMPUTE_UNITS // (_pow2(num_seqs) * kv_heads))
+    want = -(-compute_units() // (_pow2(num_seqs) * kv_heads))
     most = max(1, _pow2(max_ctx, KEYS_PER_WORKGROUP) // KEYS_PER_WORKGROUP)
     return max(1, min(want, most, MAX_KEY_SPLITS))
 
@@ -90,7 +98,7 @@ def portion_splits(workgroups: int, mean_keys: int) -> int:
     launch to twice the compute units, each worth 256 keys or more on average."""
     if workgroups <= 0:
         return 1
-    return max(1, min(SMALL_WORKGROUPS_AT_ONCE // workgroups, mean_keys // KEYS_PER_WORKGROUP, MAX_KEY_SPLITS))
+    return max(1, min(2 * compute_units() // workgroups, mean_keys // KEYS_PER_WORKGROUP, MAX_KEY_SPLITS))
 
 
 def heavy_first(work):
@@ -177,7 +185,7 @@ class PagedAttention(Mixer):
     @property
     def plan_key(self):
         s = self.spec
-        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim)
+        return ("paged_attention", s.num_heads, s.num_kv_heads, s.head_dim, s.window)
 
     def prepare(self, shape) -> None:
         """Decides once per step and head geometry how attention is launched:
@@ -211,7 +219,8 @@ class PagedAttention(Mixer):
                 # over 4: 2,048 queries in 67 to 77 us against 92, 4,096 the same either way;
                 # at 40 over 8: 1,024 in 37 against 48, 2,048 in 118 against 98.
                 small_count = int((-(-portions // (QUERY_TILE * small_tiles))).sum())
-                if small_count * hkv <= SMALL_WORKGROUPS_AT_ONCE:
+                # (two workgroups of 8 wavefronts fit on a compute unit)
+                if small_count * hkv <= 2 * compute_units():
                     plan.small, tiles = True, small_tiles
             seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE * tiles)
             # the keys an entry's last query reads: where its portion starts plus its queries
@@ -226,7 +235,8 @@ class PagedAttention(Mixer):
             plan.kernel = "tiles"
             seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE)
         plan.count = int(seqs.size)
-        plan.seq_name, plan.q0_name = f"attention_seq:{h}:{hkv}:{d}", f"attention_q0:{h}:{hkv}:{d}"
+        tag = f"{h}:{hkv}:{d}:{s.window or 0}"
+        plan.seq_name, plan.q0_name = f"attention_seq:{tag}", f"attention_q0:{tag}"
         shape.add(plan.seq_name, seqs)
         shape.add(plan.q0_name, q0)
 

@@ -95,6 +95,12 @@ class Sampler:
         n = len(rows_of_floats[0])
         turn = self._turn = 1 - getattr(self, "_turn", 0)
         if self._staging is None or self._staging[0][0].shape[1] < n:
+            if self._staging is not None:
+                # A copy kernel that is still queued reads the old buffers when it runs, and
+                # the host allocator may hand their memory to the next page-locked tensor
+                # as soon as they are dropped: they go only after their last readers.
+                for _, read in self._staging:
+                    read.synchronize()
             width = max(64, 2 * n)
             self._staging = [(torch.empty(3, width, dtype=torch.float32, pin_memory=True), torch.cuda.Event())
                              for _ in range(2)]

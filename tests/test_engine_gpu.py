@@ -7,6 +7,7 @@ import random
 import pytest
 import torch
 
+from .compare import TOL, GreedyCheck
 from .plain.model import PlainModel, softmax_sample_reference
 from .tiny import CONFIGS, PAGE_SIZES, make_model_dir
 
@@ -26,24 +27,11 @@ def prompts_for(name, lengths, seed=0):
     return [[rng.choice([t for t in range(vocab) if t not in eos]) for _ in range(n)] for n in lengths]
 
 
-def check_against_plain(plain, prompt, generated, gap, first_logits=None):
-    """Every generated token is the plain model's argmax, unless the plain
-    model's two best logits are closer than `gap` (bfloat16 near-ties; the
-    reference's tests/test_paged.py:88-99 tests the same way)."""
-    seq = list(prompt)
-    for i, tok in enumerate(generated):
-        row = plain.logits(seq)[-1]
-        if int(row.argmax()) != tok:
-            top2 = row.topk(2).values
-            assert gap > 0 and float(top2[0] - top2[1]) < gap, (
-                f"token {i}: engine chose {tok}, plain argmax {int(row.argmax())} at a clear margin"
-            )
-        seq.append(tok)
-
-
 @pytest.mark.parametrize(
     "name, lengths, new, budget",
-    [("A", [5, 11, 17], 8, 512), ("B", [1, 9, 30, 64], 12, 16), ("C", [3, 50, 28], 40, 24)],
+    [("A", [5, 11, 17], 8, 512), ("A_untied", [5, 11, 17], 24, 512), ("B", [1, 9, 30, 64], 12, 16),
+     ("C", [3, 50, 28], 40, 24),
+     ("D", [2, 70, 33, 120], 60, 48)],
 )
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_greedy_generation_through_the_entry_point(name, lengths, new, budget, dtype, model_root):
@@ -56,11 +44,10 @@ def test_greedy_generation_through_the_entry_point(name, lengths, new, budget, d
               max_tokens_per_step=budget)
     outs = llm.generate(prompts, SamplingParams(max_new_tokens=new, ignore_eos=True))
     assert [len(o) for o in outs] == [new] * len(prompts)
+    check = GreedyCheck(plain, dtype)  # float32: identical greedy tokens
     for prompt, out in zip(prompts, outs):
-        if dtype == "float32":
-            assert out == plain.greedy(prompt, new)  # identical greedy tokens
-        else:
-            check_against_plain(plain, prompt, out, gap=0.05 * float(plain.logits(prompt).abs().max()))
+        check.request(prompt, out)
+    check.finish()
     assert llm.engine.cache.num_free == llm.engine.cache.num_pages  # tests/test_paged.py:102-103
     assert llm.engine.cache.slots.num_free == llm.engine.cache.slots.num_slots
 
@@ -136,19 +123,31 @@ def test_when_pages_run_out_the_newest_request_is_preempted_and_recomputes(model
     assert tight.cache.num_free == 12 and not tight.has_work
 
 
-def test_prefix_sharing_changes_nothing_but_the_work(model_root):
+@pytest.mark.parametrize("dtype, page", [("float32", 8), ("bfloat16", 16)])
+def test_prefix_sharing_changes_nothing_but_the_work(model_root, dtype, page):
+    """bfloat16 at page size 16 runs the matrix-instruction attention kernels: a
+    request that finds its prefix in the cache computes the rest as a portion
+    that starts inside the sequence, over pages that another request wrote."""
     from shrike_amd import SamplingParams
     from shrike_amd.engine.llm_engine import LLMEngine
 
-    model_dir = make_model_dir("B", model_root, mode="unit")
+    model_dir = make_model_dir("B", model_root, dtype=dtype, mode="unit")
     common = prompts_for("B", [40], seed=6)[0]
     prompts = [common + tail for tail in ([5, 6, 7], [8], [9, 10, 11, 12, 13])]
-    sp = SamplingParams(max_new_tokens=6, ignore_eos=True)
-    off = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64, enable_prefix_caching=False)
+    sp = SamplingParams(max_new_tokens=6 if dtype == "float32" else 30, ignore_eos=True)
+    off = LLMEngine(str(model_dir), dtype=dtype, block_size=page, num_kv_blocks=64, enable_prefix_caching=False)
     want = [off.generate([p], sp)[0] for p in prompts]
-    on = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64)
+    on = LLMEngine(str(model_dir), dtype=dtype, block_size=page, num_kv_blocks=64)
     got = [on.generate([p], sp)[0] for p in prompts]
-    assert got == want
+    if dtype == "float32":
+        assert got == want
+    else:  # another cutting of the prompt may round another way: both are judged by the plain model
+        plain = PlainModel(model_dir)
+        for outs in (want, got):
+            check = GreedyCheck(plain, dtype)
+            for prompt, out in zip(prompts, outs):
+                check.request(prompt, out)
+            check.finish()
     assert on.metrics()["prefix_cache_hit_rate"] > 0.5 and off.metrics()["prefix_cache_hit_rate"] == 0
 
 
@@ -159,7 +158,7 @@ def test_long_decoding_and_first_tokens(model_root):
     from shrike_amd.engine.loading import load_model
     from shrike_amd.engine.runner import ModelRunner, StepEntry
 
-    for dtype, tol in (("float32", 1e-4), ("bfloat16", 3e-2)):
+    for dtype, tol in TOL.items():
         model_dir = make_model_dir("C", model_root, dtype=dtype, mode="unit")
         plain = PlainModel(model_dir)
         model, rt, cfg = load_model(model_dir, dtype)
@@ -181,8 +180,9 @@ def test_long_decoding_and_first_tokens(model_root):
         cache.check([])
 
 
-@pytest.mark.parametrize("dtype, tol, streamed", [("float32", 1e-4, False), ("bfloat16", 3e-2, False),
-                                                  ("bfloat16", 3e-2, True)])
+@pytest.mark.parametrize("dtype, tol, streamed", [("float32", TOL["float32"], False),
+                                                  ("bfloat16", TOL["bfloat16"], False),
+                                                  ("bfloat16", TOL["bfloat16"], True)])
 def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol, streamed, monkeypatch):
     """A 10,000-token prompt in portions of up to 4,096 tokens (the later ones
     read keys far back, through block tables of more than 600 pages), then six
@@ -231,30 +231,37 @@ def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol, streamed, monk
     cache.check([])
 
 
-def test_overlapped_steps_change_no_token(model_root, tmp_path):
+@pytest.mark.parametrize("dtype, page", [("float32", 8), ("bfloat16", 16)])
+def test_overlapped_steps_change_no_token(model_root, tmp_path, dtype, page):
     """The next decode step is launched before the host has read this step's tokens.
     With a fifth of all token ids ending a sequence, requests end at steps that
     nobody can foresee, and some are aborted while a step that holds them is
     already running: every request still yields exactly what an engine that does
-    not overlap yields for it alone, greedy or drawn."""
+    not overlap yields for it alone, greedy or drawn.  In bfloat16 (page size 16:
+    the matrix-instruction attention kernels, graphs and steps in flight together)
+    a row's bits depend on the batch it runs in, so every request is greedy and is
+    judged by the plain model instead: its tokens are the plain argmax but for a
+    few near-ties, and it ends at its first end-of-sequence token or at its length."""
     from shrike_amd import SamplingParams
     from shrike_amd.engine.llm_engine import LLMEngine
     from shrike_amd.weights import write_model_folder
 
-    cfg = dict(CONFIGS["B"], eos_token_id=list(range(3, CONFIGS["B"]["vocab_size"], 5)))
-    model_dir = write_model_folder(cfg, tmp_path / "many_ends", seed=5, mode="unit")
+    exact = dtype == "float32"
+    eos = list(range(3, CONFIGS["B"]["vocab_size"], 5))
+    cfg = dict(CONFIGS["B"], eos_token_id=eos)
+    model_dir = write_model_folder(cfg, tmp_path / "many_ends", seed=5, mode="unit", dtype=dtype)
     rng = random.Random(21)
     jobs = []
     for i in range(24):
         prompt = prompts_for("B", [rng.randint(1, 40)], seed=300 + i)[0]
         jobs.append((prompt, SamplingParams(max_new_tokens=rng.randint(1, 40), top_p=0.95, seed=i,
-                                            temperature=0.0 if i % 3 else 0.9)))
-    alone = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=64,
+                                            temperature=0.9 if exact and i % 3 == 0 else 0.0)))
+    alone = LLMEngine(str(model_dir), dtype=dtype, block_size=page, num_kv_blocks=64,
                       enable_prefix_caching=False, overlap_steps=False)
     want = [alone.generate([p], sp)[0] for p, sp in jobs]
     assert 4 < sum(len(w) < sp.max_new_tokens for w, (_, sp) in zip(want, jobs)) < 24
 
-    engine = LLMEngine(str(model_dir), dtype="float32", block_size=8, num_kv_blocks=80, max_running=8)
+    engine = LLMEngine(str(model_dir), dtype=dtype, block_size=page, num_kv_blocks=80, max_running=8)
     assert engine.config.overlap_steps
     got, ids, pending, aborted, overlapped = {}, {}, list(range(len(jobs))), set(), 0
     while pending or engine.has_work:
@@ -272,9 +279,19 @@ def test_overlapped_steps_change_no_token(model_root, tmp_path):
             got.setdefault(ids[o.req_id], []).append(o.token_id)
         engine.cache.check([r.cache for r in engine.scheduler.running if r.cache is not None])
     assert overlapped > 10 and aborted
-    for i, w in enumerate(want):
-        mine = got.get(i, [])
-        assert mine == (w[: len(mine)] if i in aborted else w), f"request {i}"
+    if exact:
+        for i, w in enumerate(want):
+            mine = got.get(i, [])
+            assert mine == (w[: len(mine)] if i in aborted else w), f"request {i}"
+    else:
+        check = GreedyCheck(PlainModel(model_dir), dtype)
+        for i, (prompt, sp) in enumerate(jobs):
+            mine = got.get(i, [])
+            check.request(prompt, mine)
+            assert not set(mine[:-1]) & set(eos), f"request {i} went on after an end-of-sequence token"
+            if i not in aborted:
+                assert mine and (mine[-1] in eos or len(mine) == sp.max_new_tokens), f"request {i}"
+        check.finish()
     assert engine.cache.num_free == 80 and not engine.scheduler.running
     engine.cache.check([])
 
@@ -484,16 +501,18 @@ def test_bfloat16_generation_survives_preemption(model_root):
     from shrike_amd import SamplingParams
     from shrike_amd.engine.llm_engine import LLMEngine
 
-    model_dir = make_model_dir("A", model_root, dtype="bfloat16", mode="unit")
+    model_dir = make_model_dir("A_untied", model_root, dtype="bfloat16", mode="unit")
     plain = PlainModel(model_dir)
     prompts = prompts_for("A", [9, 14, 6, 11], seed=5)
     tight = LLMEngine(str(model_dir), dtype="bfloat16", block_size=4, num_kv_blocks=12,
                       max_tokens_per_step=7, enable_prefix_caching=False)
     got = tight.generate(prompts, SamplingParams(max_new_tokens=20, ignore_eos=True))
     assert tight.metrics()["preemptions"] > 0
+    check = GreedyCheck(plain, "bfloat16")
     for prompt, out in zip(prompts, got):
         assert len(out) == 20
-        check_against_plain(plain, prompt, out, gap=0.05 * float(plain.logits(prompt).abs().max()))
+        check.request(prompt, out)
+    check.finish()
     assert tight.cache.num_free == 12 and not tight.has_work
     tight.cache.check([])
 

@@ -831,21 +831,25 @@ def test_rope_kv_store_adds_up_a_split_product(ops, n, splits):
      (16, 2, 64, 16, 100), (3, 1, 128, 48, None), (16, 1, 32, 16, None), (12, 1, 64, 32, 50),
      (40, 8, 128, 16, None)],
 )
-@pytest.mark.parametrize("small, nsplit", [(False, 1), (True, 1), (True, 3), (False, 8)])
-def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window, small, nsplit):
+@pytest.mark.parametrize("small, nsplit, singles", [(False, 1, 0), (True, 1, 0), (True, 3, 0), (False, 8, 0),
+                                                    (True, 3, 5), (False, 8, 5), (False, 1, 3)])
+def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size, window, small, nsplit, singles):
     """The prefill kernel that shares each chunk of keys among the query heads of a
     key/value head: 1 to 16 heads per group, portions of 2 to 200 tokens, in
     workgroups of 16 wavefronts and of 8 (`small`), every entry's keys in one
     workgroup or shared among 3 or 8 (more shares than some entries have chunks
-    of keys: the last ones find nothing to do)."""
+    of keys: the last ones find nothing to do).  `singles`: that many sequences
+    with one token each come first in the step, as in a step that mixes decoding
+    with prompt portions; the kernel is told where the prompt tokens begin
+    (first_token) and must leave the single tokens' rows alone."""
     torch.manual_seed(20)
     dtype = torch.bfloat16
     tiles = ops.attention_prefill_shared_tiles(heads, kv_heads, head_dim, small)
     assert tiles == (8 if small else 16) // (heads // kv_heads)
     if tiles == 0:
         pytest.skip("more query heads per key/value head than the small workgroup has wavefronts")
-    seq_lens = [2, 200, 16, 17, 90, 33, 130]
-    starts = [0, 60, 5, 100, 0, 31, 7]
+    seq_lens = [1] * singles + [2, 200, 16, 17, 90, 33, 130]
+    starts = [9, 40, 0, 77, 16][:singles] + [0, 60, 5, 100, 0, 31, 7]
     ctx = [s + l for s, l in zip(starts, seq_lens)]
     n = sum(seq_lens)
     num_pages = sum(-(-c // page_size) for c in ctx) + 5
@@ -857,6 +861,8 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
         cu.append(cu[-1] + l)
     wg_seq, wg_q0 = [], []
     for s, l in enumerate(seq_lens):
+        if s < singles:
+            continue  # the decode kernel's rows
         for q0 in range(0, l, 16 * tiles):
             wg_seq.append(s)
             wg_q0.append(q0)
@@ -866,13 +872,14 @@ def test_attention_prefill_shared_mfma(ops, heads, kv_heads, head_dim, page_size
     i32 = lambda x: torch.tensor(x, dtype=torch.int32, device="cuda")  # noqa: E731
     out = torch.full((n, heads * head_dim), float("nan"), device="cuda", dtype=dtype)
     scale = head_dim**-0.5
-    partial = torch.full((n * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
+    partial = torch.full(((n - singles) * heads * nsplit * (head_dim + 2),), float("nan"), device="cuda")
     ops.attention_prefill_shared(dev(q).view(n, -1), out, len(wg_seq), heads, kv_heads, head_dim, i32(cu), i32(ctx),
                                  i32(wg_seq), i32(wg_q0), tables, k_pool, v_pool, page_size, window, scale,
-                                 small=small, partial=partial, nsplit=nsplit)
+                                 small=small, partial=partial, nsplit=nsplit, first_token=singles)
     want = reference_attention(q.double(), k_pool, v_pool, tables, seq_lens, starts, page_size, window, scale)
-    assert not torch.isnan(out.float()).any()
-    close(out.view(n, heads, head_dim), want, dtype, scale=1.0)
+    assert torch.isnan(out[:singles].float()).all()  # the single tokens' rows were not touched
+    assert not torch.isnan(out[singles:].float()).any()
+    close(out[singles:].view(n - singles, heads, head_dim), want[singles:], dtype, scale=1.0)
 
 
 def test_attention_prefill_shared_refuses_wide_groups(ops):

@@ -97,13 +97,13 @@ def four_cuttings(model_dir, dtype, tol, ids, want):
     cache.check([])
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 1.5e-2)])
 def test_one_layer_of_the_7b_shape(dtype, tol, model_dir, reference):
     ids, want = reference
     four_cuttings(model_dir, dtype, tol, ids, want)
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 1.5e-2)])
 def test_one_layer_of_the_14b_shape(dtype, tol, tmp_path_factory):
     """Five query heads per key/value head, width 5120: the four cuttings again."""
     from shrike_amd.weights import write_model_folder
@@ -126,7 +126,7 @@ def long_reference(plain_model):
     return ids, plain_model.logits(ids, rows=rows).double()
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 1.5e-2)])
 def test_a_2048_token_prompt_and_decoding_past_context_4096(dtype, tol, model_dir, long_reference):
     """What the benchmark times, compared with the plain implementation: a
     2,048-token prompt in one step (64 chunks of keys for the last query tile),
@@ -210,4 +210,103 @@ def test_many_single_tokens_as_a_graph_and_kernel_by_kernel(model_dir, plain_mod
     for row in (0, 1, 37, 63, 64, count - 2, count - 1):
         for step in (0, 3):
             want = plain_model.logits(prompts[row] + feed[row][: step + 1], rows=[-1]).double()[0]
-            assert rel_err(replayed[step][row].cpu().double(), want) <= 3e-2, (row, step)
+            assert rel_err(replayed[step][row].cpu().double(), want) <= 1.5e-2, (row, step)
+
+
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 1.5e-2)])
+def test_decoding_requests_beside_a_portion_far_into_a_prompt(dtype, tol, tmp_path_factory, monkeypatch):
+    """One step of 32 single tokens beside a 480-token portion that starts at
+    position 1,120 of its prompt, with the 14B layer sizes: what a long prompt
+    under the 512-token budget looks like while others decode.  In bfloat16 the
+    portion's keys are shared among several workgroups whose results are merged
+    behind the single tokens' rows; the portion's rows and the riders' rows are
+    compared with the plain implementation."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+    from shrike_amd.kernels import ops
+    from shrike_amd.weights import write_model_folder
+
+    folder = tmp_path_factory.getbasetemp() / "big14"
+    if not (folder / "model.safetensors").is_file():
+        write_model_folder(dict(SHAPE_14B), folder, seed=9, mode="unit")
+    rng = random.Random(12)
+    vocab = SHAPE_14B["vocab_size"]
+    main = [rng.randrange(vocab) for _ in range(1600)]
+    riders = [[rng.randrange(vocab) for _ in range(rng.choice([1, 2, 15, 16, 17, 100, 333]) + 1)]
+              for _ in range(32)]
+    plain = PlainModel(folder, dtype=torch.float32)
+    main_rows = [1120, 1121, 1135, 1136, 1300, 1407, 1598, 1599]
+    want_main = plain.logits(main, rows=main_rows).double()
+    checked_riders = [0, 7, 19, 31]
+    want_riders = torch.stack([plain.logits(riders[i], rows=[-1]).double()[0] for i in checked_riders])
+
+    seen = []
+    launch = ops.attention_prefill_shared
+
+    def spy(*args, **kwargs):
+        seen.append((kwargs.get("nsplit", 1), kwargs.get("first_token", 0)))
+        return launch(*args, **kwargs)
+
+    monkeypatch.setattr(ops, "attention_prefill_shared", spy)
+    model, rt, _ = load_model(folder, dtype)
+    cache = CacheManager(model.cache_specs(), 16, 100 + 32 * 22, enable_prefix_caching=False)
+    cache.allocate(rt.dtype, rt.device)
+    for g in cache.groups:
+        g.k_tensor.fill_(float("nan"))
+        g.v_tensor.fill_(float("nan"))
+    runner = ModelRunner(model, cache, rt)
+    seq = cache.new_sequence()
+    cache.append(seq, 0, 1120)
+    runner.step([StepEntry(seq, main[:1120], 0, [])])
+    rider_seqs = [cache.new_sequence() for _ in riders]
+    warm = []
+    for s, ids in zip(rider_seqs, riders):
+        cache.append(s, 0, len(ids) - 1)
+        warm.append(StepEntry(s, ids[:-1], 0, []))
+    runner.step(warm)
+    seen.clear()
+    entries = [StepEntry(seq, main[1120:], 1120, [r - 1120 for r in main_rows])]  # the portion first:
+    cache.append(seq, 1120, 480)
+    for s, ids in zip(rider_seqs, riders):  # the step function puts the single tokens in front itself
+        cache.append(s, len(ids) - 1, 1)
+        entries.append(StepEntry(s, [ids[-1]], len(ids) - 1, [0]))
+    out = runner.step(entries).cpu().double()
+    assert out.shape[0] == len(main_rows) + 32 and torch.isfinite(out).all()
+    if dtype == "bfloat16":  # one launch for the layer: keys shared, 32 single tokens in front
+        assert seen and all(nsplit > 1 and first == 32 for nsplit, first in seen), seen
+    assert rel_err(out[: len(main_rows)], want_main) <= tol
+    got_riders = torch.stack([out[len(main_rows) + i] for i in checked_riders])
+    assert rel_err(got_riders, want_riders) <= tol
+    for s in [seq] + rider_seqs:
+        cache.free(s)
+    cache.check([])
+
+
+def test_two_layers_of_the_7b_shape_generate_the_plain_tokens(tmp_path_factory):
+    """Greedy generation through the entry point with two layers of the 7B sizes:
+    in float32 every token is the plain implementation's, prompts cut by a token
+    budget of 24; in bfloat16 but for a few near-ties."""
+    from shrike_amd import LLM, SamplingParams
+    from shrike_amd.weights import write_model_folder
+
+    from .compare import GreedyCheck
+
+    folder = write_model_folder(dict(SHAPE, num_hidden_layers=2), tmp_path_factory.mktemp("big2") / "m",
+                                seed=13, mode="unit")
+    plain = PlainModel(folder, dtype=torch.float32)
+    rng = random.Random(14)
+    prompts = [[rng.randrange(SHAPE["vocab_size"]) for _ in range(n)] for n in (40, 7)]
+    for dtype in ("float32", "bfloat16"):
+        llm = LLM(str(folder), dtype=dtype, block_size=16, num_kv_blocks=16, max_tokens_per_step=24)
+        outs = llm.generate(prompts, SamplingParams(max_new_tokens=6, ignore_eos=True))
+        check = GreedyCheck(plain, dtype)
+        for prompt, out in zip(prompts, outs):
+            assert len(out) == 6
+            check.request(prompt, out)
+        if dtype == "float32":
+            assert check.excused == 0
+        else:
+            assert check.excused <= 2
+        del llm
+        torch.cuda.empty_cache()

@@ -42,7 +42,7 @@ def test_odd_shapes(name):
         plain = PlainModel(model_dir)
         ids = torch.randint(0, case["vocab_size"], (90,), generator=torch.Generator().manual_seed(1)).tolist()
         want = plain.logits(ids)
-        for dtype, tol in (("float32", 1e-4), ("bfloat16", 3e-2)):
+        for dtype, tol in (("float32", 1e-4), ("bfloat16", 1.5e-2)):
             model, rt, _ = load_model(model_dir, dtype)
             for page_size in (16, 4):
                 cache = CacheManager(model.cache_specs(), page_size, 64, enable_prefix_caching=False)

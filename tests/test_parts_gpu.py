@@ -98,7 +98,7 @@ def test_norm_part(dtype):
     total = resid.double() + pending.to(dtype).double()
     assert hidden.pending is None and torch.allclose(hidden.resid.cpu().double(), total, atol=1e-6)
     want = plain.rms_norm(total, w.double(), 2e-4)
-    assert (out.cpu().double() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 3e-2)
+    assert (out.cpu().double() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -116,7 +116,7 @@ def test_feed_forward_part(dtype):
     out = part.forward(part_context(5, dtype), x.cuda())
     want = plain.swiglu(x.double(), w["mlp.gate_proj.weight"].double(), w["mlp.up_proj.weight"].double(),
                         w["mlp.down_proj.weight"].double())
-    assert (out.cpu().double() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 3e-2) * want.abs().max()
+    assert (out.cpu().double() - want).abs().max() <= (1e-5 if dtype == torch.float32 else 1.5e-2) * want.abs().max()
 
 
 def test_position_part_gives_the_reference_frequencies():
@@ -152,7 +152,7 @@ def test_attention_part_and_block(dtype):
     got = step_whole(runner, cache, ids, cuts=[9, 1, 11])
     cfg = plain.PlainConfig(48, 88, 1, 4, 2, 16, 97, 1e-5, 1e4, False)
     want = plain.forward(cfg, {k: v.double() for k, v in w.items()}, ids)
-    assert plain.rel_err(got, want) <= (1e-5 if dtype == torch.float32 else 3e-2)
+    assert plain.rel_err(got, want) <= (1e-5 if dtype == torch.float32 else 1.5e-2)
 
 
 # ------------------------------------------------------------- the order is data

@@ -39,6 +39,29 @@ def test_rope_is_a_complex_rotation_on_the_half_split_pairing():
     assert torch.allclose(pair(got), pair(x), atol=1e-12)
 
 
+def test_rope_frequencies_are_a_geometric_sequence_from_one_down():
+    """The rotation rates, written out as numbers rather than recomputed from the
+    expression under test (shrike/models/qwen.py:80): pair i turns by
+    theta**(-2i/d) per position, so for theta = 10^4 and d = 16 the rates are
+    10**(-i/2), and for theta = 10^6 and d = 32 each is 10**-0.375 times the one
+    before, the last 10**-5.625.  An exponent of i/d, of 2i/(d-2) or an order
+    from slow to fast fails this."""
+    cos, sin = plain.rope_tables(torch.tensor([1]), 16, 10000.0)
+    rates = torch.atan2(sin[0, :8], cos[0, :8]).double()
+    want = torch.tensor([1.0, 0.31622776601683794, 0.1, 0.031622776601683794, 0.01,
+                         0.0031622776601683794, 0.001, 0.00031622776601683794], dtype=torch.float64)
+    assert torch.allclose(rates, want, rtol=1e-6, atol=0)
+    assert torch.equal(cos[0, :8], cos[0, 8:]) and torch.equal(sin[0, :8], sin[0, 8:])  # both halves alike
+    cos, sin = plain.rope_tables(torch.tensor([1]), 32, 1e6)
+    rates = torch.atan2(sin[0, :16], cos[0, :16]).double()
+    assert abs(float(rates[0]) - 1.0) < 1e-6 and abs(float(rates[15]) / 2.3713737056616554e-06 - 1) < 1e-5
+    assert torch.allclose(rates[1:] / rates[:-1], torch.full((15,), 0.42169650342858224, dtype=torch.float64),
+                          rtol=1e-5)
+    # position scales the angle: 1,000 positions turn the slowest pair of the first table by 0.316 rad
+    cos, sin = plain.rope_tables(torch.tensor([1000]), 16, 10000.0)
+    assert abs(float(torch.atan2(sin[0, 7], cos[0, 7])) - 0.31622776601683794) < 1e-5
+
+
 def test_rope_scores_depend_only_on_distance():
     d, theta = 32, 1e6
     q, k = torch.randn(1, 1, d, dtype=torch.float64), torch.randn(1, 1, d, dtype=torch.float64)
@@ -154,3 +177,35 @@ def test_attention_of_the_last_queries_alone():
         whole = plain.causal_attention(q, k, v, window)
         for first in (0, 1, 17, 22):
             assert torch.allclose(plain.causal_attention(q[first:], k, v, window, first=first), whole[first:], atol=1e-13)
+
+
+def test_a_one_token_sequence_written_out_with_library_routines(tmp_path):
+    """With one token there is one key: softmax gives weight 1, position 0 rotates
+    nothing, and attention returns the value projection (bias included) of the
+    token itself, each key/value head repeated for its group of query heads.  The
+    whole model is then a few library calls (shrike/models/qwen.py:111-125, 131-136,
+    147-150, 190-192), written here without any function of the plain implementation:
+    a missing value bias, a bias on the output projection, a norm after instead of
+    before a part, or a residual taken from the normed input would all differ."""
+    for name in ("A", "B", "C"):
+        m = plain.PlainModel(make_model_dir(name, tmp_path, mode="unit"))
+        cfg, w = m.cfg, m.weights
+        tok = 17
+        x = w["model.embed_tokens.weight"][tok].double()
+        group = cfg.num_heads // cfg.num_kv_heads
+        for i in range(cfg.num_layers):
+            pre = f"model.layers.{i}."
+            h = F.rms_norm(x, x.shape, w[pre + "input_layernorm.weight"].double(), cfg.rms_norm_eps)
+            v = F.linear(h, w[pre + "self_attn.v_proj.weight"].double(), w[pre + "self_attn.v_proj.bias"].double())
+            attn = v.view(cfg.num_kv_heads, 1, cfg.head_dim).expand(-1, group, -1).reshape(-1)
+            x = x + F.linear(attn, w[pre + "self_attn.o_proj.weight"].double())
+            h = F.rms_norm(x, x.shape, w[pre + "post_attention_layernorm.weight"].double(), cfg.rms_norm_eps)
+            act = F.silu(F.linear(h, w[pre + "mlp.gate_proj.weight"].double())) * F.linear(
+                h, w[pre + "mlp.up_proj.weight"].double())
+            x = x + F.linear(act, w[pre + "mlp.down_proj.weight"].double())
+        x = F.rms_norm(x, x.shape, w["model.norm.weight"].double(), cfg.rms_norm_eps)
+        out = w.get("lm_head.weight", w["model.embed_tokens.weight"]).double()
+        want = F.linear(x, out)
+        got = m.logits([tok])[0].double()
+        assert torch.allclose(got, want, rtol=1e-9, atol=1e-9), name
+        assert not any(k.endswith(("o_proj.bias", "gate_proj.bias", "up_proj.bias", "down_proj.bias")) for k in w)

@@ -1,7 +1,10 @@
 """bin/trace_run against the plain implementation: the same requests whole,
 with the last 32 tokens one by one, in portions of changing size, and mixed
 with other requests over so few pages that they are used again; in float32 and
-in bfloat16; for three tiny configurations."""
+in bfloat16; for four tiny configurations (D runs the matrix-instruction
+attention kernels with a window, so that pages a window has passed are given
+back, poisoned and handed out again under those kernels and under the graphs
+of its single-token steps)."""
 
 import random
 
@@ -16,10 +19,12 @@ from .traces import (TraceBuilder, changing_portions, check_pages, last_one_by_o
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [5, 11, 17, 70, 45], "B": [1, 9, 30, 64, 100], "C": [3, 40, 97, 65, 130]}
+LENGTHS = {"A": [5, 11, 17, 70, 45], "B": [1, 9, 30, 64, 100], "C": [3, 40, 97, 65, 130],
+           "D": [6, 50, 130, 90, 200]}
 # float32: rel err <= 1e-4 is the engine's stated bound.  bfloat16: 8 bits of
-# mantissa, a handful of roundings per layer.
-TOL = {"float32": 1e-4, "bfloat16": 3e-2}
+# mantissa, a handful of roundings per layer; the worst error seen over some
+# thousands of seeds of these models is 8e-3 of the largest logit.
+TOL = {"float32": 1e-4, "bfloat16": 1.5e-2}
 
 
 def requests_for(name: str) -> dict[str, list[int]]:
@@ -34,7 +39,7 @@ def model_root(tmp_path_factory):
 
 
 # each tiny model at its own page size (4, 8, 16) and at 16, the size that serving uses
-CASES = sorted({(name, size) for name in "ABC" for size in (PAGE_SIZES[name], 16)})
+CASES = sorted({(name, size) for name in "ABCD" for size in (PAGE_SIZES[name], 16)})
 
 
 @pytest.mark.parametrize("mode", ["reference", "unit"])

@@ -124,7 +124,7 @@ def test_resumed_request_recomputes_prompt_and_generated_tokens_in_portions():
     sched.add(a)
     sched.postprocess(sched.schedule())
     a.token_ids += [50, 51, 52]  # generated before a preemption
-    sched._preempt_for(None)
+    sched._preempt_newest()
     assert a.num_computed_tokens == 0 and a.cache is None
     batch = sched.schedule()
     assert ids(batch) == [(a.req_id, 6)]

@@ -173,7 +173,7 @@ def test_the_writer_and_the_loader_know_the_toy_by_its_config_alone(toy):
     assert len(model.cache_specs()) == 4 and all(s is not None for s in model.cache_specs())
 
 
-@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 3e-2)])
+@pytest.mark.parametrize("dtype, tol", [("float32", 1e-4), ("bfloat16", 1.5e-2)])
 def test_the_toy_steps_and_generates_like_its_plain_form(toy, dtype, tol):
     from shrike_amd import LLM, SamplingParams
 
@@ -189,7 +189,7 @@ def test_the_toy_steps_and_generates_like_its_plain_form(toy, dtype, tol):
             row = plain_logits(weights, seq)[-1]
             if int(row.argmax()) != tok:
                 top2 = row.topk(2).values
-                assert dtype == "bfloat16" and float(top2[0] - top2[1]) < 0.05 * float(row.abs().max())
+                assert dtype == "bfloat16" and float(top2[0] - top2[1]) < 0.03 * float(row.abs().max())
             seq.append(tok)
     # and the logits themselves, through the step function, portions beside a single token
     from shrike_amd.cache import CacheManager

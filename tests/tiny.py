@@ -1,6 +1,7 @@
 """Tiny configurations of the architecture for tests.  A and B differ in every
 size and option; C has an explicit head_dim (heads * head_dim != hidden) and a
-window on its later layers."""
+window on its later layers; D has a head size that the matrix-instruction
+attention kernels take (64) and a window on all layers but the first."""
 
 from __future__ import annotations
 
@@ -63,9 +64,33 @@ TINY_C = {
     "max_window_layers": 2,
 }
 
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-SEEDS = {"A": 11, "B": 23, "C": 37}
-PAGE_SIZES = {"A": 4, "B": 8, "C": 16}
+TINY_D = {
+    "architectures": ["Qwen2ForCausalLM"],
+    "hidden_size": 160,
+    "intermediate_size": 296,
+    "num_hidden_layers": 3,
+    "num_attention_heads": 4,
+    "num_key_value_heads": 2,
+    "head_dim": 64,
+    "vocab_size": 389,
+    "rope_theta": 200000.0,
+    "rms_norm_eps": 2e-5,
+    "tie_word_embeddings": False,
+    "torch_dtype": "float32",
+    "use_sliding_window": True,
+    "sliding_window": 40,
+    "max_window_layers": 1,
+}
+
+# A with an output matrix of its own.  With "unit" weights the tied table is N(0, 1), and
+# a token's logit for itself (its embedding's squared length) towers over all others:
+# greedy generation of tied A says little about the layers in between, so tests of
+# generated tokens take this variant; logits are compared on A itself.
+TINY_A_UNTIED = dict(TINY_A, tie_word_embeddings=False)
+
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "A_untied": TINY_A_UNTIED}
+SEEDS = {"A": 11, "B": 23, "C": 37, "D": 41, "A_untied": 11}
+PAGE_SIZES = {"A": 4, "B": 8, "C": 16, "D": 16, "A_untied": 4}
 
 
 def make_model_dir(name: str, root=None, dtype: str = "float32", mode: str = "reference") -> Path:
