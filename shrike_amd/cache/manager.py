@@ -2,13 +2,12 @@
 one pool per group of layers with the same need, and slots for per-request
 state of fixed size.
 
-Layers whose mixers ask for the same PagedKVSpec form a group; a group has its
-own pool of pages, its own device tensors (keys in slabs of 32 elements,
-``[layers, pages, kv_heads, head_dim / 32, page_size, 32]``; values transposed,
-``[layers, pages, kv_heads, head_dim, page_size]``, so that the keys of a page
-are contiguous for every element) and, per request, its own block table.  A
-group with a window gives pages back as soon as no later query
-can reach them (table entry -1); all pages come back when the request ends.
+Layers whose mixers ask for the same PagedSpec form a group; a group has its
+own pool of pages, its own device tensors (whatever the spec lists per page,
+each as ``[layers, pages + 1, *its shape for one page]``: what a page holds and
+how it is laid out is the mixer's business, not the manager's) and, per request,
+its own block table.  A group with a window gives pages back as soon as no later
+query can reach them (table entry -1); all pages come back when the request ends.
 Layers whose mixers ask for a StateSpec form state groups: a tensor
 ``[layers, slots, *shape]`` indexed by the request's state slot.  Every request
 holds one slot, whether or not any layer has state.
@@ -22,7 +21,7 @@ from __future__ import annotations
 
 from dataclasses import dataclass, field
 
-from ..parts.base import PagedKVSpec, StateSpec
+from ..parts.base import PagedSpec, StateSpec
 from .pages import PageError, PagePool, SlotPool
 
 
@@ -43,8 +42,9 @@ class LayerCache:
     group: int  # index into ctx.block_tables / ctx.state tensors
     owned: bool  # False: reads the cache another schedule position writes
     page_size: int = 0
-    k_pool: object = None
-    v_pool: object = None
+    # name -> this layer's slice [pages + 1, *shape of one page] of each tensor the
+    # mixer's PagedSpec lists (empty where no device memory was allocated)
+    pools: dict = field(default_factory=dict)
     window: int | None = None
     state: object = None  # [slots, *shape] for a StateSpec layer
     # the same memory with one slot more, [slots + 1, *shape]: the padding rows of
@@ -54,12 +54,11 @@ class LayerCache:
 
 
 class PageGroup:
-    def __init__(self, spec: PagedKVSpec, num_pages: int):
+    def __init__(self, spec: PagedSpec, num_pages: int):
         self.spec = spec
         self.layers: list[int] = []  # schedule positions that own a cache of this group
         self.pool = PagePool(num_pages)
-        self.k_tensor = None
-        self.v_tensor = None
+        self.tensors: dict = {}  # name -> [layers, pages + 1, *shape of one page]
 
 
 class StateGroup:
@@ -90,7 +89,7 @@ class CacheManager:
         for pos, spec in enumerate(layer_specs):
             if spec is None:
                 continue
-            if isinstance(spec, PagedKVSpec):
+            if isinstance(spec, PagedSpec):
                 family, groups, make = "pages", self.groups, lambda s: PageGroup(s, num_pages)
             elif isinstance(spec, StateSpec):
                 family, groups, make = "state", self.state_groups, StateGroup
@@ -118,30 +117,28 @@ class CacheManager:
     # ----------------------------------------------------------- device memory
 
     def bytes_per_page(self, elem_size: int) -> int:
-        """Bytes that one page id costs over all groups and layers."""
-        return sum(
-            len(g.layers) * 2 * self.page_size * g.spec.num_kv_heads * g.spec.head_dim * elem_size
-            for g in self.groups
-        )
+        """Bytes that one page id costs over all groups and layers; `elem_size` is
+        that of the compute dtype, which tensors without a dtype of their own have."""
+        import torch
+
+        total = 0
+        for g in self.groups:
+            for t in g.spec.tensors:
+                size = elem_size if t.dtype is None else torch.empty(0, dtype=getattr(torch, t.dtype)).element_size()
+                total += len(g.layers) * t.numel(self.page_size) * size
+        return total
 
     def allocate(self, dtype, device) -> None:
         import torch
 
         for g in self.groups:
-            s = g.spec
             # one page more than the pool hands out: page `num_pages` is where the
-            # padding rows of a fixed-size (graph) batch put their keys and values
-            # keys of a page and head in slabs of 32 elements (whole rows where the head
-            # size is no multiple of 32): what the attention kernels' operand loads want
-            slab = 32 if s.head_dim % 32 == 0 else s.head_dim
-            g.k_tensor = torch.zeros(
-                len(g.layers), self.num_pages + 1, s.num_kv_heads, s.head_dim // slab, self.page_size, slab,
-                dtype=dtype, device=device,
-            )
-            g.v_tensor = torch.zeros(
-                len(g.layers), self.num_pages + 1, s.num_kv_heads, s.head_dim, self.page_size,
-                dtype=dtype, device=device,
-            )
+            # padding rows of a fixed-size (graph) batch put what they write
+            for t in g.spec.tensors:
+                g.tensors[t.name] = torch.zeros(
+                    len(g.layers), self.num_pages + 1, *t.shape(self.page_size),
+                    dtype=dtype if t.dtype is None else getattr(torch, t.dtype), device=device,
+                )
         for g in self.state_groups:
             g.padded = torch.zeros(
                 len(g.layers), self.slots.num_slots + 1, *g.spec.shape,
@@ -157,8 +154,7 @@ class CacheManager:
             g = self.groups[gi]
             return LayerCache(
                 group=gi, owned=not reader, page_size=self.page_size,
-                k_pool=None if g.k_tensor is None else g.k_tensor[li],
-                v_pool=None if g.v_tensor is None else g.v_tensor[li],
+                pools={name: t[li] for name, t in g.tensors.items()},
                 window=g.spec.window,
             )
         g = self.state_groups[gi]

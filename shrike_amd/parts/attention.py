@@ -8,7 +8,7 @@ import numpy as np
 import torch
 
 from ..kernels import ops
-from .base import Mixer, PagedKVSpec, ParamSpec, build_part, register_mixer
+from .base import PAGE, Mixer, PagedSpec, PageTensor, ParamSpec, build_part, register_mixer
 
 QUERY_TILE = 16  # queries per tile of the MFMA kernels for prompt portions
 COMPUTE_UNITS = 256  # of an MI355X; compute_units() asks the device that is there
@@ -28,6 +28,22 @@ def compute_units() -> int:
         _UNITS = (torch.cuda.get_device_properties(torch.cuda.current_device()).multi_processor_count
                   if torch.cuda.is_available() else COMPUTE_UNITS)
     return _UNITS
+
+
+def kv_cache_spec(num_kv_heads: int, head_dim: int, window: int | None = None) -> PagedSpec:
+    """The cache of grouped-query attention, laid out for this file's kernels: per
+    page and key/value head the keys in slabs of 32 elements, [head_dim / 32,
+    page_size, 32] (a wavefront's operand load for the matrix instruction then
+    touches whole cache lines: 64 bytes from each of four consecutive keys; one
+    slab of head_dim elements where head_dim is no multiple of 32), and the values
+    transposed, [head_dim, page_size] (the keys of a page side by side for every
+    element, which is the operand layout of V^T)."""
+    slab = ops.key_slab(head_dim)
+    return PagedSpec(
+        tensors=(PageTensor("k", (num_kv_heads, head_dim // slab, PAGE, slab)),
+                 PageTensor("v", (num_kv_heads, head_dim, PAGE))),
+        window=window,
+    )
 
 
 def _pow2(n: int, floor: int = 1) -> int:
@@ -146,7 +162,7 @@ class PagedAttention(Mixer):
 
     def cache_spec(self):
         s = self.spec
-        return PagedKVSpec(s.num_kv_heads, s.head_dim, s.window)
+        return kv_cache_spec(s.num_kv_heads, s.head_dim, s.window)
 
     def check(self, runtime):
         s = self.spec
@@ -250,14 +266,14 @@ class PagedAttention(Mixer):
                                "(the step function calls prepare() on every part)")
         q = qkv[:, : h * d]
         if not plan.mfma:
-            ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.k_pool,
-                          cache.v_pool, cache.page_size, s.window, s.scale)
+            ops.attention(q, out, h, hkv, d, ctx.positions, ctx.token_seq, tables, cache.pools["k"],
+                          cache.pools["v"], cache.page_size, s.window, s.scale)
             return
         if ctx.num_decode:
             partial = ctx.buffer("attn_partial", (ctx.num_decode * h * plan.nsplit * (d + 2),),
                                  torch.float32)
             ops.attention_decode(q, out, ctx.num_decode, h, hkv, d, ctx.positions, tables,
-                                 cache.k_pool, cache.v_pool, cache.page_size, s.window, s.scale,
+                                 cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale,
                                  partial, plan.nsplit, plan.streaming)
         if plan.kernel == "shared":
             partial = None
@@ -267,13 +283,13 @@ class PagedAttention(Mixer):
                                      (prompt_tokens * h * plan.portion_splits * (d + 2),), torch.float32)
             ops.attention_prefill_shared(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                          ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
-                                         cache.k_pool, cache.v_pool, cache.page_size, s.window,
+                                         cache.pools["k"], cache.pools["v"], cache.page_size, s.window,
                                          s.scale, small=plan.small, partial=partial,
                                          nsplit=plan.portion_splits, first_token=plan.first_token)
         elif plan.kernel == "tiles":
             ops.attention_prefill(q, out, plan.count, h, hkv, d, ctx.cu_q, ctx.ctx_lens,
                                   ctx.extras[plan.seq_name], ctx.extras[plan.q0_name], tables,
-                                  cache.k_pool, cache.v_pool, cache.page_size, s.window, s.scale)
+                                  cache.pools["k"], cache.pools["v"], cache.page_size, s.window, s.scale)
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:
         s = self.spec
@@ -296,7 +312,7 @@ class PagedAttention(Mixer):
         tables = ctx.block_tables[cache.group]
         ops.rope_kv_store(
             qkv, s.num_heads, s.num_kv_heads, s.head_dim, rot_dim, inv_freq, ctx.positions,
-            ctx.token_seq, tables, cache.k_pool, cache.v_pool, cache.page_size,
+            ctx.token_seq, tables, cache.pools["k"], cache.pools["v"], cache.page_size,
             write_kv=cache.owned, split_sum=split_sum,
         )
         attn = ctx.buffer("attn_out", (n, s.num_heads * s.head_dim), ctx.dtype)

@@ -52,14 +52,44 @@ class ParamSpec:
     optional: bool = False
 
 
-@dataclass(frozen=True)
-class PagedKVSpec:
-    """Cache need of a mixer: keys and values per token, kept for all earlier
-    tokens (window None) or for the last `window` of them."""
+PAGE = "page"  # in a PageTensor's dims: the place of the page size
 
-    num_kv_heads: int
-    head_dim: int
+
+@dataclass(frozen=True)
+class PageTensor:
+    """One tensor that a mixer keeps for every page of a sequence.  `dims` is the
+    shape of one page's part of it, ints and PAGE (the page size, which only the
+    engine's options fix); the layout within a page is the mixer's own business
+    and that of its kernels.  `dtype` None: the compute dtype."""
+
+    name: str
+    dims: tuple
+    dtype: str | None = None
+
+    def shape(self, page_size: int) -> tuple[int, ...]:
+        return tuple(page_size if d == PAGE else int(d) for d in self.dims)
+
+    def numel(self, page_size: int) -> int:
+        n = 1
+        for d in self.shape(page_size):
+            n *= d
+        return n
+
+
+@dataclass(frozen=True)
+class PagedSpec:
+    """Cache need of a mixer: something per token, kept in pages, for all earlier
+    tokens (window None) or for the last `window` of them.  The cache manager
+    allocates every listed tensor as [layers, pages + 1, *dims] and hands a
+    layer its slice under the tensor's name; it knows nothing else about them."""
+
+    tensors: tuple[PageTensor, ...]
     window: int | None = None
+
+    def __post_init__(self):
+        names = [t.name for t in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a paged cache needs tensors with distinct names, got {names}")
 
 
 @dataclass(frozen=True)
@@ -134,7 +164,7 @@ class Mixer(Part):
     state_graph_safe = False
 
     def cache_spec(self):
-        """PagedKVSpec, StateSpec or None."""
+        """PagedSpec, StateSpec or None."""
         return None
 
     def forward(self, ctx, x: torch.Tensor, cache) -> torch.Tensor:

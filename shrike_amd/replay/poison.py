@@ -1,7 +1,7 @@
 """Poisoning of cache pages that no request holds.
 
 A page that is free, or was never used, is filled with NaN in every layer of
-its group.  Whatever reads it (a stale block table, a key beyond a request's
+its group, in every floating-point tensor that the group's mixers keep per page.  Whatever reads it (a stale block table, a key beyond a request's
 length, a page that a window has already given back) then shows up as NaN in
 the logits, instead of as the plausible numbers a finished request left there.
 The fills are ordinary tensor fills on the pool's slices, outside any HIP graph.
@@ -19,16 +19,17 @@ class PagePoisoner:
     def poison_everything(self) -> None:
         """Before the first step: every page of every group, the spare page included."""
         for g in self.cache.groups:
-            g.k_tensor.fill_(float("nan"))
-            g.v_tensor.fill_(float("nan"))
+            for t in g.tensors.values():
+                if t.is_floating_point():
+                    t.fill_(float("nan"))
 
     def poison_pages(self, group: int, pages) -> None:
         pages = sorted(set(int(p) for p in pages))
         if not pages:
             return
-        g = self.cache.groups[group]
-        g.k_tensor[:, pages] = float("nan")
-        g.v_tensor[:, pages] = float("nan")
+        for t in self.cache.groups[group].tensors.values():
+            if t.is_floating_point():
+                t[:, pages] = float("nan")
 
     def held(self, seq: SequenceCache) -> list[list[int]]:
         """The pages a request holds now, per group."""

@@ -7,10 +7,11 @@ import random
 import pytest
 
 from shrike_amd.cache import CacheManager, PageError, PagePool
-from shrike_amd.parts.base import PagedKVSpec, StateSpec
+from shrike_amd.parts import kv_cache_spec
+from shrike_amd.parts.base import StateSpec
 
-FULL = PagedKVSpec(num_kv_heads=2, head_dim=16)
-WIN = PagedKVSpec(num_kv_heads=2, head_dim=16, window=6)
+FULL = kv_cache_spec(num_kv_heads=2, head_dim=16)
+WIN = kv_cache_spec(num_kv_heads=2, head_dim=16, window=6)
 
 
 def manager(num_pages=8, page_size=4, specs=(FULL, FULL), **kw):
@@ -260,25 +261,25 @@ def test_poisoned_free_pages_show_through_a_shifted_table():
     shifted to a free page, or to a page the request gave back, meets NaN."""
     import torch
 
-    from shrike_amd.parts import PagedKVSpec
+    from shrike_amd.parts import kv_cache_spec
     from shrike_amd.replay.poison import PagePoisoner
 
-    cache = CacheManager([PagedKVSpec(2, 32), PagedKVSpec(2, 32, window=8)], 4, 12, enable_prefix_caching=False)
+    cache = CacheManager([kv_cache_spec(2, 32), kv_cache_spec(2, 32, window=8)], 4, 12, enable_prefix_caching=False)
     cache.allocate(torch.float32, "cpu")
     poisoner = PagePoisoner(cache)
     poisoner.poison_everything()
-    assert all(torch.isnan(g.k_tensor).all() and torch.isnan(g.v_tensor).all() for g in cache.groups)
+    assert all(torch.isnan(g.tensors["k"]).all() and torch.isnan(g.tensors["v"]).all() for g in cache.groups)
 
     def write(seq, group, first, last):
         g = cache.groups[group]
         for p in range(first, last):
             page = seq.tables[group][p // 4]
-            g.k_tensor[0, page, :, :, p % 4, :] = float(p)
-            g.v_tensor[0, page, :, :, p % 4] = float(p)
+            g.tensors["k"][0, page, :, :, p % 4, :] = float(p)
+            g.tensors["v"][0, page, :, :, p % 4] = float(p)
 
     def read(table, group, first, last):
         g = cache.groups[group]
-        return torch.stack([g.k_tensor[0, table[p // 4], :, :, p % 4, :].flatten() for p in range(first, last)])
+        return torch.stack([g.tensors["k"][0, table[p // 4], :, :, p % 4, :].flatten() for p in range(first, last)])
 
     a, b = cache.new_sequence(), cache.new_sequence()
     cache.append(a, 0, 10)
@@ -302,7 +303,7 @@ def test_poisoned_free_pages_show_through_a_shifted_table():
     write(a, 1, 10, 12)
     assert cache.trim(a, 12) == 1 and a.tables[1][0] == -1
     assert poisoner.poison_released(before, a) == [[], [old_first]]
-    assert torch.isnan(cache.groups[1].k_tensor[0, old_first]).all()
+    assert torch.isnan(cache.groups[1].tensors["k"][0, old_first]).all()
     assert torch.isfinite(read(a.tables[1], 1, 5, 12)).all()
 
     # b ends: its pages are poisoned, a's are not
@@ -310,7 +311,7 @@ def test_poisoned_free_pages_show_through_a_shifted_table():
     cache.free(b)
     assert poisoner.poison_released(before) == before
     for gi, pages in enumerate(before):
-        assert torch.isnan(cache.groups[gi].v_tensor[0, pages]).all()
+        assert torch.isnan(cache.groups[gi].tensors["v"][0, pages]).all()
     assert torch.isfinite(read(a.tables[0], 0, 0, 12)).all()
     cache.free(a)
     cache.check([])

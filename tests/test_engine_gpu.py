@@ -209,8 +209,8 @@ def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol, streamed, monk
     cache = CacheManager(model.cache_specs(), 16, 640, enable_prefix_caching=False)
     cache.allocate(rt.dtype, rt.device)
     for g in cache.groups:  # a slot that is read before it is written shows up as NaN
-        g.k_tensor.fill_(float("nan"))
-        g.v_tensor.fill_(float("nan"))
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
     runner = ModelRunner(model, cache, rt)
     seq = cache.new_sequence()
     got = []

@@ -141,8 +141,8 @@ def test_a_2048_token_prompt_and_decoding_past_context_4096(dtype, tol, model_di
     cache = CacheManager(model.cache_specs(), 16, 300, enable_prefix_caching=False)
     cache.allocate(rt.dtype, rt.device)
     for g in cache.groups:  # a slot that is read before it is written shows up as NaN
-        g.k_tensor.fill_(float("nan"))
-        g.v_tensor.fill_(float("nan"))
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
     runner = ModelRunner(model, cache, rt)
     seq = cache.new_sequence()
     cache.append(seq, 0, 2048)
@@ -253,8 +253,8 @@ def test_decoding_requests_beside_a_portion_far_into_a_prompt(dtype, tol, tmp_pa
     cache = CacheManager(model.cache_specs(), 16, 100 + 32 * 22, enable_prefix_caching=False)
     cache.allocate(rt.dtype, rt.device)
     for g in cache.groups:
-        g.k_tensor.fill_(float("nan"))
-        g.v_tensor.fill_(float("nan"))
+        for t in g.tensors.values():
+            t.fill_(float("nan"))
     runner = ModelRunner(model, cache, rt)
     seq = cache.new_sequence()
     cache.append(seq, 0, 1120)

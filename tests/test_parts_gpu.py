@@ -145,9 +145,9 @@ def test_attention_part_and_block(dtype):
     names = sorted(p.name.split("self_attn.")[1] for p in mixer.params())
     assert names == ["k_proj.bias", "k_proj.weight", "o_proj.weight", "q_proj.bias", "q_proj.weight",
                      "v_proj.bias", "v_proj.weight"]
-    from shrike_amd.parts import PagedKVSpec
+    from shrike_amd.parts import kv_cache_spec
 
-    assert mixer.cache_spec() == PagedKVSpec(2, 16, None)
+    assert mixer.cache_spec() == kv_cache_spec(2, 16, None)
     ids = torch.randint(0, 97, (21,), generator=torch.Generator().manual_seed(1)).tolist()
     got = step_whole(runner, cache, ids, cuts=[9, 1, 11])
     cfg = plain.PlainConfig(48, 88, 1, 4, 2, 16, 97, 1e-5, 1e4, False)
@@ -644,3 +644,143 @@ def test_toy_embedding_and_head_are_parts_like_the_others():
     want = want_for(ids)
     assert plain.rel_err(step_whole(runner, cache, ids), want) <= 1e-5
     assert plain.rel_err(step_whole(runner, cache, ids, [6, 1, 1, 2, 19]), want) <= 1e-5
+
+
+# ------------------- a toy paged mixer whose cache is one latent vector per token
+
+
+@dataclass(frozen=True)
+class LatentSpec:
+    """Attention over one shared latent per token: c_t = W_c x_t is all that is
+    cached; y_t = W_o sum_j softmax_j(q_t . c_j / sqrt(r)) c_j over the tokens j
+    up to t (the last `window` of them), q_t = W_q x_t."""
+
+    kind: ClassVar[str] = "toy_latent"
+    latent: int
+    window: int | None = None
+
+
+def define_toy_latent_mixer():
+    from shrike_amd.parts import PAGE, Mixer, PagedSpec, PageTensor, ParamSpec, register_mixer
+
+    class LatentMixer(Mixer):
+        graph_safe = False  # its forward walks the sequences on the host
+
+        def params(self):
+            r, h = self.spec.latent, self.width
+            return [ParamSpec(f"{self.name}.q_proj.weight", (r, h)), ParamSpec(f"{self.name}.c_proj.weight", (r, h)),
+                    ParamSpec(f"{self.name}.o_proj.weight", (h, r))]
+
+        def cache_spec(self):
+            # one tensor per page, in float32 whatever the compute dtype: a layout of its own
+            return PagedSpec((PageTensor("latent", (PAGE, self.spec.latent), "float32"),), self.spec.window)
+
+        def load(self, tensors, runtime):
+            self.wq, self.wc, self.wo = (tensors[f"{self.name}.{n}_proj.weight"].float() for n in "qco")
+
+        def forward(self, ctx, x, cache):
+            pool, ps = cache.pools["latent"], cache.page_size  # [pages + 1, page_size, latent]
+            tables = ctx.block_tables[cache.group].long()
+            pos, seq = ctx.positions.long(), ctx.token_seq.long()
+            q, c = x.float() @ self.wq.t(), x.float() @ self.wc.t()
+            if cache.owned:
+                pool[tables[seq, pos // ps], pos % ps] = c
+            out = torch.empty_like(q)
+            start = 0
+            for s, (n, length) in enumerate(zip(ctx.q_lens, ctx.ctx_lens_host)):
+                first = 0 if self.spec.window is None else max(0, length - n - self.spec.window + 1)
+                lo = first // ps  # pages before it may have been given back (table entry -1)
+                pages = tables[s, lo : -(-length // ps)]
+                keys = pool[pages].reshape(-1, self.spec.latent)[: length - lo * ps]
+                j = torch.arange(lo * ps, length, device=x.device)[None, :]
+                p = pos[start : start + n, None]
+                seen = (j <= p) if self.spec.window is None else (j <= p) & (j > p - self.spec.window)
+                scores = (q[start : start + n] @ keys.t()) * self.spec.latent**-0.5
+                out[start : start + n] = scores.masked_fill(~seen, float("-inf")).softmax(-1) @ keys
+                start += n
+            return (out @ self.wo.t()).to(x.dtype)
+
+    register_mixer("toy_latent", LatentMixer)
+
+
+@pytest.mark.parametrize("window", [None, 11])
+def test_toy_paged_mixer_with_one_latent_per_token_keeps_its_own_layout(window):
+    """A mixer whose pages hold a single tensor of its own shape and dtype is
+    registered, given pages, stepped in several cuttings beside ordinary attention
+    layers, and survives the poisoning of every page that no request holds, without
+    a change to the cache manager, the step function or the poisoner."""
+    from shrike_amd.engine.runner import StepEntry
+    from shrike_amd.parts import PAGE, PagedSpec, PageTensor
+    from shrike_amd.replay.poison import PagePoisoner
+
+    define_toy_latent_mixer()
+    base = small_spec()
+    toy_block = replace(base.blocks[1], mixer=LatentSpec(latent=24, window=window), mixer_name="latent")
+    spec = replace(base, blocks=(base.blocks[0], toy_block))
+    w = cpu_weights(spec, seed=6)
+    runner, model, cache = make_runner(spec, w, page_size=4, num_pages=24)
+    assert model.cache_specs()[1] == PagedSpec((PageTensor("latent", (PAGE, 24), "float32"),), window)
+    assert len(cache.groups) == 2  # attention's keys and values; the toy's latents
+    latents = cache.groups[1].tensors
+    assert list(latents) == ["latent"] and latents["latent"].shape == (1, 25, 4, 24)
+    assert latents["latent"].dtype == torch.float32
+    kv_bytes = 2 * 4 * 2 * 16 * 4  # keys and values of a page: 4 tokens, 2 heads of 16, float32
+    assert cache.bytes_per_page(4) == kv_bytes + 4 * 24 * 4
+    assert runner.use_graphs is False
+
+    def want_for(ids):
+        cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
+        wd = {k: v.double() for k, v in w.items()}
+        n = len(ids)
+        cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+        x = plain.decoder_layer(cfg, wd, 0, wd["model.embed_tokens.weight"][torch.tensor(ids)], cos, sin)
+        p = "model.layers.1"
+        h = plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5)
+        q, c = h @ wd[f"{p}.latent.q_proj.weight"].t(), h @ wd[f"{p}.latent.c_proj.weight"].t()
+        # plain attention with one head whose keys and values are the same vectors
+        att = plain.causal_attention(q[:, None], c[:, None], c[:, None], window)
+        x = x + att[:, 0] @ wd[f"{p}.latent.o_proj.weight"].t()
+        h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
+        x = x + plain.swiglu(h, wd[f"{p}.mlp.gate_proj.weight"], wd[f"{p}.mlp.up_proj.weight"], wd[f"{p}.mlp.down_proj.weight"])
+        return plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+
+    poisoner = PagePoisoner(cache)
+    poisoner.poison_everything()
+    assert torch.isnan(latents["latent"]).all()
+    g = torch.Generator().manual_seed(4)
+    a = torch.randint(0, 97, (41,), generator=g).tolist()
+    b = torch.randint(0, 97, (23,), generator=g).tolist()
+    wa, wb = want_for(a), want_for(b)
+    assert plain.rel_err(step_whole(runner, cache, a), wa) <= 1e-5
+    poisoner.poison_everything()  # the request is gone: all its pages are poisoned again
+    assert plain.rel_err(step_whole(runner, cache, a, [7, 2, 1, 1, 19, 11]), wa) <= 1e-5
+    poisoner.poison_everything()
+    # two requests side by side, a portion of one beside single tokens of the other; the
+    # windowed group gives pages back on the way, and they are poisoned at once
+    sa, sb = cache.new_sequence(), cache.new_sequence()
+    rows = {}
+    pa = pb = 0
+    for na, nb in [(9, 1), (1, 1), (20, 2), (1, 13), (10, 6)]:
+        entries = []
+        for seq, ids, p, n, name in ((sa, a, pa, na, "a"), (sb, b, pb, nb, "b")):
+            cache.append(seq, p, n)
+            entries.append(StepEntry(seq, ids[p : p + n], p, list(range(n))))
+        before = [poisoner.held(sa), poisoner.held(sb)]
+        out = runner.step(entries).cpu().double()
+        assert torch.isfinite(out).all()
+        for i in range(na):
+            rows[("a", pa + i)] = out[i]
+        for i in range(nb):
+            rows[("b", pb + i)] = out[na + i]
+        pa, pb = pa + na, pb + nb
+        for seq, p, held in ((sa, pa, before[0]), (sb, pb, before[1])):
+            cache.trim(seq, p)
+            poisoner.poison_released(held, seq)
+    assert pa == 41 and pb == 23
+    assert plain.rel_err(torch.stack([rows[("a", i)] for i in range(41)]), wa) <= 1e-5
+    assert plain.rel_err(torch.stack([rows[("b", i)] for i in range(23)]), wb) <= 1e-5
+    if window:
+        assert -1 in sa.tables[1] and -1 not in sa.tables[0]  # only the toy's group has a window
+    cache.free(sa)
+    cache.free(sb)
+    cache.check([])

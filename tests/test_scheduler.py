@@ -9,9 +9,9 @@ import pytest
 from shrike_amd.cache import CacheManager
 from shrike_amd.engine.request import Request, SamplingParams, Status
 from shrike_amd.engine.scheduler import Scheduler
-from shrike_amd.parts.base import PagedKVSpec
+from shrike_amd.parts import kv_cache_spec
 
-SPEC = PagedKVSpec(num_kv_heads=1, head_dim=16)
+SPEC = kv_cache_spec(num_kv_heads=1, head_dim=16)
 
 
 def req(tokens, max_new=8) -> Request:
@@ -169,7 +169,7 @@ def test_prefix_hit_shortens_the_first_portion():
 
 
 def test_window_pages_come_back_during_a_long_request():
-    win = PagedKVSpec(num_kv_heads=1, head_dim=16, window=5)
+    win = kv_cache_spec(num_kv_heads=1, head_dim=16, window=5)
     cm = cache(4, 4, specs=(win,))
     sched = Scheduler(cm, max_tokens_per_step=4)
     a = req(range(40), max_new=1)  # 10 pages worth of prompt through a pool of 4
