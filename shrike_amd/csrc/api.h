@@ -27,11 +27,6 @@ int shk_copy_words(const int32_t* src, int32_t* dst, int n, const int32_t* patch
 int shk_gather_rows(const int32_t* src, long long ld, int src_rows, const int32_t* index, int32_t* dst,
                     int rows, int width, void* stream);
 
-// Reads `bytes` bytes from p (16-byte aligned) with `workgroups` workgroups of 512
-// threads and keeps nothing: a kernel that needs them next finds them in the caches
-// between the compute units and memory.  sink may be null.
-int shk_touch(const void* p, long long bytes, int workgroups, int32_t* sink, void* stream);
-
 // Zeroes `bytes` bytes from dst, which must be 4-byte aligned (a fill kernel:
 // it may be recorded into a HIP graph).
 int shk_zero_bytes(void* dst, long long bytes, void* stream);

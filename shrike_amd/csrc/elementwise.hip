@@ -189,25 +189,6 @@ __global__ void __launch_bounds__(256) zero_bytes_kernel(uint8_t* __restrict__ d
   if (blockIdx.x == 0 && threadIdx.x < bytes - words * 4) dst[words * 4 + threadIdx.x] = 0;
 }
 
-// Reads `n16` 16-byte units from p and keeps nothing: what it read then lies in the
-// caches between the compute units and memory for the kernel that needs it next.
-__global__ void __launch_bounds__(512)
-    touch_kernel(const uint4* __restrict__ p, long long n16, int32_t* __restrict__ sink) {
-  const long long stride = static_cast<long long>(gridDim.x) * blockDim.x;
-  uint32_t acc = 0;
-  long long i = blockIdx.x * static_cast<long long>(blockDim.x) + threadIdx.x;
-  for (; i + 3 * stride < n16; i += 4 * stride) {
-    const uint4 a = p[i], b = p[i + stride], c = p[i + 2 * stride], d = p[i + 3 * stride];
-    acc ^= a.x ^ a.w ^ b.x ^ b.w ^ c.x ^ c.w ^ d.x ^ d.w;
-  }
-  for (; i < n16; i += stride) {
-    const uint4 a = p[i];
-    acc ^= a.x ^ a.w;
-  }
-  // never true for memory that holds bfloat16 weights; it keeps the loads alive
-  if (acc == 0x7fc00001u && sink != nullptr) *sink = 1;
-}
-
 }  // namespace shk
 
 using namespace shk;
@@ -238,17 +219,6 @@ extern "C" int shk_gather_rows(const int32_t* src, long long ld, int src_rows, c
   gather_rows_kernel<<<dim3(per_row, rows), 256, 0, static_cast<hipStream_t>(stream)>>>(src, ld, index, dst,
                                                                                        width);
   SHK_LAUNCH_CHECK("gather_rows");
-  return 0;
-}
-
-extern "C" int shk_touch(const void* p, long long bytes, int workgroups, int32_t* sink, void* stream) {
-  SHK_REQUIRE(bytes >= 0 && workgroups >= 1 && workgroups <= 65535, "touch: bad sizes bytes=%lld workgroups=%d",
-              bytes, workgroups);
-  if (bytes < 16) return 0;
-  SHK_REQUIRE(p && reinterpret_cast<uintptr_t>(p) % 16 == 0, "touch: p must be 16-byte aligned");
-  touch_kernel<<<workgroups, 512, 0, static_cast<hipStream_t>(stream)>>>(static_cast<const uint4*>(p),
-                                                                        bytes / 16, sink);
-  SHK_LAUNCH_CHECK("touch");
   return 0;
 }
 

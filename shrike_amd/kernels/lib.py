@@ -20,7 +20,6 @@ _SIGNATURES = {
     "shk_copy_words": [_P, _P, _I, _P, _I, _I, _P],
     "shk_gather_rows": [_P, c_longlong, _I, _P, _P, _I, _I, _P],
     "shk_zero_bytes": [_P, c_longlong, _P],
-    "shk_touch": [_P, c_longlong, _I, _P, _P],
     "shk_embed": [_P, _I, _P, _P, _I, _I, _I, _P],
     "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "shk_silu_mul": [_P, _P, _I, _I, _I, _P],

@@ -90,19 +90,6 @@ def gather_rows(src: torch.Tensor, index: torch.Tensor, dst: torch.Tensor) -> No
                                  _dev(dst, "dst"), dst.shape[0], dst.shape[1], _stream()))
 
 
-def touch(t: torch.Tensor, workgroups: int = 256, nbytes: int | None = None, offset: int = 0) -> None:
-    """Reads `nbytes` bytes of a contiguous device tensor from byte `offset` on (all of
-    it by default) and keeps nothing: the next kernel that needs them finds them in
-    the caches on the way to memory."""
-    if not t.is_contiguous():
-        raise KernelError("touch: expected a contiguous tensor")
-    total = t.numel() * t.element_size()
-    nbytes = total - offset if nbytes is None else nbytes
-    if offset < 0 or offset % 16 or nbytes < 0 or offset + nbytes > total:
-        raise KernelError("touch: the range does not lie within the tensor (offset in steps of 16 bytes)")
-    check(load().shk_touch(_dev(t, "t") + offset, nbytes, workgroups, None, _stream()))
-
-
 def zero_(t: torch.Tensor) -> None:
     """Fills a contiguous device tensor with zero bytes by a kernel of the library."""
     if not t.is_contiguous():

@@ -198,7 +198,7 @@ def test_a_context_of_ten_thousand_tokens(model_root, dtype, tol, streamed, monk
         monkeypatch.setattr(attention, "STREAMING_FROM_BYTES", 0)
     flags = []
     launch = ops.attention_decode
-    monkeypatch.setattr(ops, "attention_decode", lambda *a: (flags.append(a[15]), launch(*a))[1])
+    monkeypatch.setattr(ops, "attention_decode", lambda *a, **kw: (flags.append(a[15]), launch(*a, **kw))[1])
 
     model_dir = make_model_dir("B", model_root, dtype=dtype, mode="unit")
     ids = prompts_for("B", [10006], seed=9)[0]
