@@ -15,9 +15,13 @@ decode step's unavoidable HBM reads (every weight once, the live requests'
 cache) against 8 TB/s, and against the bandwidth that a plain device copy
 reaches on this GPU (`achievable`); `prefill.achievable_frac` prices the prompt
 against the rate of the engine's own 4096^3 product; `points` holds batch 1 and
-64, and the same batches at a context near 4,000; `breakdown_us` is the decode
-step's time by kernel, from events around every launch of a step that runs
-kernel by kernel.
+64, the same batches at a context near 4,000, a 2,048-token prompt taken in
+portions under the reference's 512-token budget, batch 8 at a context of 16,000,
+and, with the layer sizes of two larger published models (`config.points_shapes`),
+a step of 32 decodes beside a prompt portion (14B) and decode at batch 64 (32B);
+`breakdown_us` is the decode step's time by kernel, from events around every
+launch of a step that runs kernel by kernel.  The larger models' points are left
+out when the run has already taken two minutes.
 """
 
 from __future__ import annotations
@@ -138,7 +142,9 @@ def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int,
     from shrike_amd import SamplingParams
 
     rng = random.Random(seed)
-    sampling = SamplingParams(max_new_tokens=batch + warmup + steps + 8, ignore_eos=True,
+    # the first requests decode while the later ones' prompts are taken in, portion by portion
+    prefill_steps = batch * -(-prompt_len // engine.scheduler.max_tokens_per_step)
+    sampling = SamplingParams(max_new_tokens=prefill_steps + batch + warmup + steps + 8, ignore_eos=True,
                               temperature=temperature, top_p=top_p)
     for _ in range(batch):
         engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(prompt_len)], sampling)
@@ -167,6 +173,70 @@ def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int,
         "context_end": context_end, "step_bytes": step_bytes,
         "gb_s": step_bytes / (ms * 1e-3) / 1e9,
     }
+
+
+def run_chunked_prefill(engine, cfg, seed: int, budget: int = 512) -> float:
+    """Milliseconds until a PROMPT_LEN-token prompt has its first token when the
+    scheduler cuts it into portions of `budget` tokens (the reference's default)."""
+    import torch
+
+    from shrike_amd import SamplingParams
+
+    rng = random.Random(seed + 3)
+    saved, engine.scheduler.max_tokens_per_step = engine.scheduler.max_tokens_per_step, budget
+    best = None
+    try:
+        for _ in range(2):
+            engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)],
+                               SamplingParams(max_new_tokens=1, ignore_eos=True))
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            steps = 0
+            while engine.has_work:
+                engine.step()
+                steps += 1
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            assert steps == -(-PROMPT_LEN // budget)
+            best = dt if best is None else min(best, dt)
+    finally:
+        engine.scheduler.max_tokens_per_step = saved
+    return best * 1e3
+
+
+def other_shapes(args, started: float, limit: float = 120.0) -> tuple[dict, str]:
+    """Points with the layer sizes of larger published models, each skipped once the
+    whole run has taken `limit` seconds: a step of 32 decodes beside a portion of a
+    2,048-token prompt under a 512-token budget (14B), decode at batch 64 (32B)."""
+    import torch
+
+    from shrike_amd.models.qwen2 import Qwen2Config, build_spec
+
+    points, named = {}, []
+    for shape, what in (("14b", "mixed"), ("32b", "decode")):
+        if time.perf_counter() - started > limit:
+            print(f"[bench] {shape} point skipped: the run has taken {time.perf_counter() - started:.0f}s", file=sys.stderr)
+            continue
+        cfg = Qwen2Config.from_dict(_shape(shape))
+        spec = build_spec(cfg)
+        named.append(f"{shape}: {cfg.num_hidden_layers} layers, hidden {cfg.hidden_size}, {cfg.num_attention_heads} heads "
+                     f"over {cfg.num_key_value_heads} of {cfg.head_dim}, intermediate {cfg.intermediate_size}")
+        if what == "mixed":
+            engine = make_engine(cfg, spec, 33, args.seed, budget=512)
+            mixed = run_mixed(engine, cfg, 32, 512, args.seed)
+            points["mixed_14b_ms"] = mixed["mixed_step_ms"]
+            points["decode_b32_14b_ms"] = mixed["decode_only_ms"]
+            print(f"[bench] 14B sizes, 32 decodes + a portion under a 512-token budget: {mixed}", file=sys.stderr)
+        else:
+            engine = make_engine(cfg, spec, 64, args.seed)
+            run = run_decode(engine, cfg, 64, min(args.steps, 40), args.warmup, args.seed + 64)
+            points["decode_b64_32b"] = round(run["tok_s"], 1)
+            points["decode_b64_32b_hbm_frac"] = round(run["gb_s"] / HBM_PEAK_GBS, 4)
+            print(f"[bench] 32B sizes, batch 64: {run['tok_s']:.1f} tok/s, {run['ms_per_step']:.3f} ms/step, "
+                  f"{run['gb_s']:.0f} GB/s", file=sys.stderr)
+        del engine
+        torch.cuda.empty_cache()
+    return points, "; ".join(named)
 
 
 def run_prefill(engine, cfg, seed: int, repeats: int = 3) -> dict:
@@ -335,6 +405,7 @@ def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
 
 def main() -> int:
     global CONTEXT_END
+    started = time.perf_counter()
     ap = argparse.ArgumentParser(description=__doc__.split("\n\n")[0])
     ap.add_argument("--gpus", type=int, default=int(os.environ.get("WORLD_SIZE", "1")))
     ap.add_argument("--steps", type=int, default=1900,
@@ -441,6 +512,17 @@ def main() -> int:
               f"{sampled['ms_per_step']:.3f} ms/step", file=sys.stderr)
     prefill = run_prefill(engine, cfg, args.seed)
     print(f"[bench] prefill: {prefill}", file=sys.stderr)
+    more_points = {}
+    if not args.no_points and args.shape == "7b":
+        more_points["prefill_2048_budget512_ms"] = round(run_chunked_prefill(engine, cfg, args.seed), 3)
+        print(f"[bench] 2,048-token prompt in portions of 512: {more_points['prefill_2048_budget512_ms']} ms",
+              file=sys.stderr)
+        if 8 * (16000 // PAGE_SIZE + 16) <= engine.cache.num_pages:
+            long_run = run_decode(engine, cfg, 8, min(args.steps, 40), args.warmup, args.seed + 300, 16000)
+            more_points["decode_b8_ctx16000"] = round(long_run["tok_s"], 1)
+            more_points["decode_b8_ctx16000_hbm_frac"] = round(long_run["gb_s"] / HBM_PEAK_GBS, 4)
+            print(f"[bench] batch 8 at context {long_run['context_start']:.0f}: {long_run['tok_s']:.1f} tok/s, "
+                  f"{long_run['ms_per_step']:.3f} ms/step, {long_run['gb_s']:.0f} GB/s", file=sys.stderr)
     # one batch left running for the per-kernel times
     from shrike_amd import SamplingParams
 
@@ -461,6 +543,14 @@ def main() -> int:
         prefill["mfma_tflops"] = peaks["mfma_tflops"]  # the matrix units alone, random operands
         prefill["achievable_frac"] = round(
             prefill_flops(cfg, PROMPT_LEN) / (prefill["ms"] * 1e-3) / (peaks["gemm_tflops"] * 1e12), 4)
+
+    graphs_on = bool(engine.config.graphs and engine.runner.use_graphs)
+    points_shapes = ""
+    if not args.no_points and args.shape == "7b":
+        del engine
+        torch.cuda.empty_cache()
+        extra, points_shapes = other_shapes(args, started)
+        more_points.update(extra)
 
     main_run = results[args.batch]
     line = {
@@ -496,7 +586,8 @@ def main() -> int:
             "page_size": PAGE_SIZE,
             "parallelism": "single GPU",
             "sampling": "greedy",
-            "hip_graphs": bool(engine.config.graphs and engine.runner.use_graphs),
+            "hip_graphs": graphs_on,
+            "points_shapes": points_shapes,
         },
         "prefill": prefill,
         "roofline": {
@@ -514,6 +605,7 @@ def main() -> int:
         line["points"][f"decode_b{b}_ctx4000"] = round(r["tok_s"], 1)
     if sampled:
         line["points"][f"decode_b{args.batch}_top_p"] = round(sampled["tok_s"], 1)
+    line["points"].update(more_points)
     if peaks:
         line["roofline"]["achievable"] = peaks["copy_gbs"]
         line["roofline"]["achievable_read"] = peaks["read_gbs"]

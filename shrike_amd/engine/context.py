@@ -44,8 +44,15 @@ class Workspace:
         self.keep_outgrown = keep_outgrown
         self._flat: dict[tuple[str, torch.dtype], torch.Tensor] = {}
         self._outgrown: list[torch.Tensor] = []
+        # (name, dtype, shape) -> the view that was handed out last time: a step asks for
+        # the same few dozen buffers layer after layer, and making a view costs a microsecond
+        self._views: dict[tuple, torch.Tensor] = {}
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        shape = tuple(shape)
+        view = self._views.get((name, dtype, shape))
+        if view is not None:
+            return view
         numel = 1
         for s in shape:
             numel *= s
@@ -56,7 +63,12 @@ class Workspace:
                 self._outgrown.append(flat)
             flat = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._flat[key] = flat
-        return flat[:numel].view(shape)
+            # views of the buffer that was replaced must not be handed out again
+            self._views = {k: v for k, v in self._views.items() if k[0] != name or k[1] != dtype}
+        view = flat[:numel].view(shape)
+        if len(self._views) < 4096:
+            self._views[(name, dtype, shape)] = view
+        return view
 
     def nbytes(self) -> int:
         held = list(self._flat.values()) + self._outgrown

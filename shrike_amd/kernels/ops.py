@@ -20,12 +20,17 @@ def dtype_code(dtype: torch.dtype) -> int:
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_device_index: int | None = None
 
 
 def _stream() -> int:
-    """Handle of the current HIP stream (the capture stream while a graph is recorded)."""
+    """Handle of the current HIP stream (the capture stream while a graph is recorded).
+    The engine runs on one GPU: its index is asked for once."""
+    global _device_index
+    if _device_index is None:
+        _device_index = torch.cuda.current_device()
     if _raw_stream is not None:  # a tenth of the cost of building a torch.cuda.Stream object
-        return _raw_stream(torch.cuda.current_device())
+        return _raw_stream(_device_index)
     return torch.cuda.current_stream().cuda_stream
 
 
