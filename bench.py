@@ -314,7 +314,7 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
 
     from shrike_amd.kernels import ops
 
-    names = ["embed", "add_rmsnorm", "silu_mul", "gemm", "gemm_tiled_weight", "rope_kv_store", "attention",
+    names = ["embed", "add_rmsnorm", "act_mul", "gemm", "gemm_tiled_weight", "rope_kv_store", "attention",
              "attention_decode", "attention_prefill", "attention_prefill_shared", "argmax", "sample"]
     spans: list[tuple[str, object, object]] = []
     saved = {n: getattr(ops, n) for n in names}

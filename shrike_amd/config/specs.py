@@ -52,10 +52,12 @@ class AttentionSpec:
 
 @dataclass(frozen=True)
 class SwiGLUSpec:
-    """down(silu(gate(x)) * up(x)) without biases."""
+    """down(act(gate(x)) * up(x)) without biases; act is "silu" (SwiGLU proper) or
+    "gelu_tanh" (the tanh form of GELU)."""
 
     kind: ClassVar[str] = "swiglu"
     intermediate_size: int
+    activation: str = "silu"
 
 
 @dataclass(frozen=True)

@@ -45,8 +45,9 @@ int shk_add_rmsnorm(float* resid, const void* delta, const float* weight, float 
                     int dtype, const int32_t* rows, int n, int hidden, int write_resid,
                     int delta_splits, int resid_rows, void* stream);
 
-// out[i, j] = silu(gu[i, j]) * gu[i, inter + j] for j < inter; gu is [n, 2*inter].
-int shk_silu_mul(const void* gu, void* out, int dtype, int n, int inter, void* stream);
+// out[i, j] = act(gu[i, j]) * gu[i, inter + j] for j < inter; gu is [n, 2*inter].
+// act 1: SiLU; act 2: GELU in its tanh form.
+int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act, void* stream);
 
 // out[n, m] (+)= a[n, k] @ w[m, k]^T + bias[m].  a and w have in_dtype, out has
 // out_dtype, bias is float32 or null.  lda/ldo are row strides in elements.
@@ -67,8 +68,9 @@ int shk_interleave_gate_up(const void* gate_t, const void* up_t, int m, int k, v
 
 // out[n, m] (+)= a[n, k] @ w^T + bias with w given in the tiled layout; a is
 // bfloat16 row-major with row stride lda; out is bfloat16 or float32.
-// gated: wt is an interleaved gate/up pair and out[n, m] = silu(a @ gate^T) *
-// (a @ up^T), without bias or accumulation.
+// gated != 0: wt is an interleaved gate/up pair and out[n, m] = act(a @ gate^T) *
+// (a @ up^T), without bias or accumulation; gated is the activation, 1 for SiLU,
+// 2 for GELU in its tanh form.
 // ksplit > 1 (at most 64 rows, float32 output, no bias): the k range is shared
 // by ksplit workgroups per block of weight rows and out is [ksplit][n][m], the
 // partial sums, which the kernel that reads the product adds up in order

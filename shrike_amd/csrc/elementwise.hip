@@ -1,4 +1,4 @@
-// Embedding lookup, residual add + RMSNorm, SiLU-multiply.
+// Embedding lookup, residual add + RMSNorm, gate activation times up.
 // All arithmetic is float32; storage is float32 or bfloat16.
 #include <stdarg.h>
 #include <stdio.h>
@@ -145,16 +145,19 @@ __global__ void __launch_bounds__(kNormThreads)
   }
 }
 
-// ---------------------------------------------------------------- SiLU * up
+// ------------------------------------------------------------ act(gate) * up
+// act 1: SiLU, g / (1 + exp(-g)).  act 2: the tanh form of GELU,
+// 0.5 g (1 + tanh(u)), u = sqrt(2/pi) (g + 0.044715 g^3), written as g / (1 + exp(-2u)).
 
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter) {
+__global__ void act_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int act) {
   const size_t row = blockIdx.y;
   const int j = blockIdx.x * blockDim.x + threadIdx.x;
   if (j >= inter) return;
   const float g = to_float(gu[row * 2 * inter + j]);
   const float u = to_float(gu[row * 2 * inter + inter + j]);
-  const float s = g / (1.f + expf(-g));
+  const float x = act == 2 ? 2.f * 0.7978845608028654f * (g + 0.044715f * g * g * g) : g;
+  const float s = g / (1.f + expf(-x));
   out[row * inter + j] = from_float<T>(s * u);
 }
 
@@ -298,20 +301,21 @@ extern "C" int shk_add_rmsnorm(float* resid, const void* delta, const float* wei
   return 0;
 }
 
-extern "C" int shk_silu_mul(const void* gu, void* out, int dtype, int n, int inter, void* stream) {
-  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "silu_mul: unknown dtype %d", dtype);
-  SHK_REQUIRE(n >= 0 && inter > 0, "silu_mul: bad sizes n=%d inter=%d", n, inter);
+extern "C" int shk_act_mul(const void* gu, void* out, int dtype, int n, int inter, int act, void* stream) {
+  SHK_REQUIRE(dtype == kF32 || dtype == kBF16, "act_mul: unknown dtype %d", dtype);
+  SHK_REQUIRE(act == 1 || act == 2, "act_mul: unknown activation %d", act);
+  SHK_REQUIRE(n >= 0 && inter > 0, "act_mul: bad sizes n=%d inter=%d", n, inter);
   if (n == 0) return 0;
-  SHK_REQUIRE(n <= 65535, "silu_mul: at most 65535 rows a call, got %d", n);
-  SHK_REQUIRE(gu && out, "silu_mul: null pointer");
+  SHK_REQUIRE(n <= 65535, "act_mul: at most 65535 rows a call, got %d", n);
+  SHK_REQUIRE(gu && out, "act_mul: null pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
   dim3 grid((inter + 255) / 256, n);
   if (dtype == kF32)
-    silu_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gu),
-                                                static_cast<float*>(out), inter);
+    act_mul_kernel<float><<<grid, 256, 0, s>>>(static_cast<const float*>(gu),
+                                                static_cast<float*>(out), inter, act);
   else
-    silu_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gu),
-                                               static_cast<bf16*>(out), inter);
-  SHK_LAUNCH_CHECK("silu_mul");
+    act_mul_kernel<bf16><<<grid, 256, 0, s>>>(static_cast<const bf16*>(gu),
+                                               static_cast<bf16*>(out), inter, act);
+  SHK_LAUNCH_CHECK("act_mul");
   return 0;
 }

@@ -63,6 +63,19 @@ struct SkinnyBatch {
 
 __device__ __forceinline__ float silu(float g) { return g / (1.f + __expf(-g)); }
 
+// The activation of a gated product's gate: kActSilu, or the tanh form of GELU,
+// 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3))) = g / (1 + exp(-2 u)).  Gated
+// kernels get the code in the argument that other products use for `accumulate`
+// (a gated product never accumulates).
+constexpr int kActSilu = 1, kActGeluTanh = 2;
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == kActGeluTanh) {
+    const float u = 0.7978845608028654f * (g + 0.044715f * g * g * g);
+    return g / (1.f + __expf(-2.f * u));
+  }
+  return silu(g);
+}
+
 template <int NB, int RB>
 __device__ __forceinline__ void skinny_load(SkinnyBatch<NB, RB>& b, const uint4* __restrict__ wrow,
                                             const bf16* __restrict__ a, int lda, int n, int k,
@@ -256,12 +269,12 @@ __global__ void __launch_bounds__(WAVES* kWave)
 #pragma unroll
       for (int w = 1; w < WAVES; ++w) up += red[w][RB - 1][b][ln][r];
     }
-    if (GATED) v = silu(v) * up;
+    if (GATED) v = gate_act(v, accumulate) * up;
     if (bias) v += bias[row];
     const size_t idx = static_cast<size_t>(token) * ldo + row;
     if (out_f32) {
       float* o = static_cast<float*>(out);
-      o[idx] = accumulate ? o[idx] + v : v;
+      o[idx] = (accumulate && !GATED) ? o[idx] + v : v;
     } else {
       static_cast<bf16*>(out)[idx] = from_float<bf16>(v);
     }
@@ -387,7 +400,7 @@ __global__ void __launch_bounds__(WAVES* kWave)
     float v[4];
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      v[r] = GATED ? silu(acc[0][b][r]) * acc[RB - 1][b][r] : acc[0][b][r];
+      v[r] = GATED ? gate_act(acc[0][b][r], accumulate) * acc[RB - 1][b][r] : acc[0][b][r];
       if (bias && row0 + r < m) v[r] += bias[row0 + r];
     }
     if (ksplit > 1) {
@@ -402,7 +415,7 @@ __global__ void __launch_bounds__(WAVES* kWave)
       float* o = static_cast<float*>(out) + idx;
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+        if (row0 + r < m) o[r] = (accumulate && !GATED) ? o[r] + v[r] : v[r];
     } else {
       bf16* o = static_cast<bf16*>(out) + idx;
       if (row0 + 3 < m && (ldo & 3) == 0) {
@@ -452,7 +465,7 @@ __device__ __forceinline__ void big_store(const f32x4 (&acc)[WM][WN], int lane, 
       float v[4];
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        v[r] = GATED ? silu(acc[i][jn][r]) * acc[i + (GATED ? 1 : 0)][jn][r]
+        v[r] = GATED ? gate_act(acc[i][jn][r], accumulate) * acc[i + (GATED ? 1 : 0)][jn][r]
                      : acc[i][jn][r] + add[GATED ? 0 : i][r];
       }
       const size_t idx = (static_cast<size_t>(share) * n + token) * ldo + row0;
@@ -460,7 +473,7 @@ __device__ __forceinline__ void big_store(const f32x4 (&acc)[WM][WN], int lane, 
         float* o = static_cast<float*>(out) + idx;
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+          if (row0 + r < m) o[r] = (accumulate && !GATED) ? o[r] + v[r] : v[r];
       } else {
         bf16* o = static_cast<bf16*>(out) + idx;
         if (row0 + 3 < m && (ldo & 3) == 0) {
@@ -1022,7 +1035,7 @@ __global__ void __launch_bounds__(16 * kWave)
         for (int b = 0; b < NB; ++b) {
           const f32x4 up = hand[((pair - first) * NB + b) * kWave + lane];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) acc[b][r] = silu(acc[b][r]) * up[r];
+          for (int r = 0; r < 4; ++r) acc[b][r] = gate_act(acc[b][r], accumulate) * up[r];
         }
       }
     }
@@ -1055,7 +1068,7 @@ __global__ void __launch_bounds__(16 * kWave)
       float* o = static_cast<float*>(out) + idx;
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (row0 + r < m) o[r] = accumulate ? o[r] + v[r] : v[r];
+        if (row0 + r < m) o[r] = (accumulate && !GATED) ? o[r] + v[r] : v[r];
     } else {
       bf16* o = static_cast<bf16*>(out) + idx;
       if (row0 + 3 < m && (ldo & 3) == 0) {
@@ -1334,6 +1347,7 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
                                           void* out, int n, int m, int k, int lda, int ldo,
                                           int out_dtype, int accumulate, int gated, int ksplit,
                                           void* stream) {
+  SHK_REQUIRE(gated >= 0 && gated <= kActGeluTanh, "gemm_bf16: unknown gate activation %d", gated);
   SHK_REQUIRE(!gated || (!accumulate && !bias), "gemm_bf16: a gated product takes no bias and does not accumulate");
   SHK_REQUIRE(ksplit >= 1 && ksplit <= 64, "gemm_bf16: ksplit %d is outside 1..64", ksplit);
   SHK_REQUIRE(ksplit == 1 || (!gated && !accumulate && !bias && out_dtype == kF32 && ldo == m),
@@ -1344,6 +1358,7 @@ extern "C" int shk_gemm_bf16_tiled_weight(const void* a, const void* wt, const f
   SHK_REQUIRE(lda >= k && ldo >= m, "gemm_bf16: row strides lda=%d ldo=%d too small", lda, ldo);
   SHK_REQUIRE(!accumulate || out_dtype == kF32, "gemm_bf16: accumulate needs a float32 output");
   if (n == 0) return 0;
+  if (gated) accumulate = gated;  // the gated kernels read the activation from this argument
   SHK_REQUIRE(a && wt && out, "gemm_bf16: null pointer");
   const int mb = (m + 15) / 16, kt = (k + 31) / 32;
   const int vec = (k % 8 == 0 && lda % 8 == 0 && (reinterpret_cast<uintptr_t>(a) % 16) == 0);

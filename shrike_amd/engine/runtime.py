@@ -47,15 +47,15 @@ class Runtime:
             return LinearWeight(gate.shape, None, tiled)
         return self.weight(torch.cat([gate, up], dim=0))
 
-    def gated_linear(self, ctx, x, w: LinearWeight, out) -> None:
-        """out = silu(x @ gate.T) * (x @ up.T).  bfloat16: one product whose
-        epilogue applies the activation; float32: product, then activation."""
+    def gated_linear(self, ctx, x, w: LinearWeight, out, activation: str = "silu") -> None:
+        """out = act(x @ gate.T) * (x @ up.T), act "silu" or "gelu_tanh".  bfloat16: one
+        product whose epilogue applies the activation; float32: product, then activation."""
         if w.tiled is not None:
-            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, gated=True)
+            ops.gemm_tiled_weight(x, w.tiled, w.rows, w.cols, out, gated=activation)
             return
         gate_up = ctx.buffer("ffn_gate_up", (x.shape[0], w.rows), self.dtype)
         ops.gemm(x, w.dense, gate_up)
-        ops.silu_mul(gate_up, out)
+        ops.act_mul(gate_up, out, activation)
 
     def linear(self, x, w: LinearWeight, out, bias=None, accumulate=False) -> None:
         """out (+)= x @ w.T + bias."""

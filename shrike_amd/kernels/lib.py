@@ -22,7 +22,7 @@ _SIGNATURES = {
     "shk_zero_bytes": [_P, c_longlong, _P],
     "shk_embed": [_P, _I, _P, _P, _I, _I, _I, _P],
     "shk_add_rmsnorm": [_P, _P, _P, _F, _P, _I, _P, _I, _I, _I, _I, _I, _P],
-    "shk_silu_mul": [_P, _P, _I, _I, _I, _P],
+    "shk_act_mul": [_P, _P, _I, _I, _I, _I, _P],
     "shk_gemm": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "shk_retile_weight": [_P, _I, _I, _P, _P],
     "shk_interleave_gate_up": [_P, _P, _I, _I, _P, _P],

@@ -147,15 +147,30 @@ def add_rmsnorm(resid, delta, weight, eps: float, out, rows=None, write_resid=Tr
     )
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
-    """out = silu(gate_up[:, :I]) * gate_up[:, I:]."""
+GATE_ACTIVATIONS = {"silu": 1, "gelu_tanh": 2}
+
+
+def activation_code(gated) -> int:
+    """0 for a product that is not gated; else the code of the gate's activation
+    (True stands for "silu")."""
+    if not gated:
+        return 0
+    name = "silu" if gated is True else gated
+    try:
+        return GATE_ACTIVATIONS[name]
+    except KeyError:
+        raise KernelError(f"gate activation must be one of {sorted(GATE_ACTIVATIONS)}, got {gated!r}") from None
+
+
+def act_mul(gate_up: torch.Tensor, out: torch.Tensor, activation: str = "silu") -> None:
+    """out = act(gate_up[:, :I]) * gate_up[:, I:]."""
     n, inter = out.shape
     if gate_up.shape != (n, 2 * inter) or not gate_up.is_contiguous() or not out.is_contiguous():
-        raise KernelError("silu_mul: gate_up must be contiguous [n, 2*inter]")
+        raise KernelError("act_mul: gate_up must be contiguous [n, 2*inter]")
     if gate_up.dtype != out.dtype:
-        raise KernelError("silu_mul: dtypes differ")
-    check(load().shk_silu_mul(_dev(gate_up, "gate_up"), _dev(out, "out"), dtype_code(out.dtype),
-                              n, inter, _stream()))
+        raise KernelError("act_mul: dtypes differ")
+    check(load().shk_act_mul(_dev(gate_up, "gate_up"), _dev(out, "out"), dtype_code(out.dtype),
+                             n, inter, activation_code(activation), _stream()))
 
 
 def gemm(a, w, out, bias=None, accumulate=False) -> None:
@@ -238,7 +253,9 @@ def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, g
     """out (+)= a @ w.T + bias with wt = retile_weight(w): up to 64 rows of a
     stream the weights once; more rows run the LDS-staged MFMA kernel (tiles of
     128 x 128 to 256 x 256, chosen by how many the product has).
-    splits > 1: out is float32 [splits, n, m] and receives partial sums."""
+    splits > 1: out is float32 [splits, n, m] and receives partial sums.
+    gated: False, or the gate's activation ("silu", "gelu_tanh"; True is "silu") for
+    an interleaved gate/up weight."""
     _rows(a, "gemm a")
     n = a.shape[0]
     if a.shape[1] != k or a.dtype != torch.bfloat16:
@@ -259,7 +276,7 @@ def gemm_tiled_weight(a, wt, m: int, k: int, out, bias=None, accumulate=False, g
             _dev(a, "a"), _dev(wt, "wt"),
             None if bias is None else _dev(bias, "bias", torch.float32),
             _dev(out, "out"), n, m, k, a.stride(0), out.stride(-2), dtype_code(out.dtype),
-            int(bool(accumulate)), int(bool(gated)), int(splits), _stream(),
+            int(bool(accumulate)), activation_code(gated), int(splits), _stream(),
         )
     )
 

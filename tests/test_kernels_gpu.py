@@ -82,15 +82,25 @@ def test_add_rmsnorm(ops, dtype, hidden, eps):
     close(out3, torch.full((1, hidden), 2.0 / math.sqrt(4.0 + eps)), dtype)
 
 
+def gate_reference(gate, activation):
+    """SiLU, or GELU in its tanh form, by the library's own routines, in float64."""
+    if activation == "silu":
+        return torch.nn.functional.silu(gate)
+    return torch.nn.functional.gelu(gate, approximate="tanh")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
 @pytest.mark.parametrize("n, inter", [(1, 172), (7, 18944), (33, 100)])
-def test_silu_mul(ops, dtype, n, inter):
+def test_act_mul(ops, dtype, n, inter, activation):
     torch.manual_seed(3)
     gu = torch.randn(n, 2 * inter) * 4
     out = torch.empty(n, inter, device="cuda", dtype=dtype)
-    ops.silu_mul(dev(gu, dtype), out)
+    ops.act_mul(dev(gu, dtype), out, activation)
     g, u = rounded(gu, dtype)[:, :inter], rounded(gu, dtype)[:, inter:]
-    close(out, g * torch.sigmoid(g) * u, dtype)
+    close(out, gate_reference(g, activation) * u, dtype)
+    with pytest.raises(Exception, match="activation"):
+        ops.act_mul(dev(gu, dtype), out, "relu")
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -749,18 +759,24 @@ def test_attention_mfma_finds_one_far_key_among_thousands(ops):
                                          (9, 100, 1700), (50, 64, 3000), (40, 16400, 1040),
                                          (64, 18944, 3584), (17, 2000, 416), (32, 66000, 64),
                                          (65, 172, 64), (300, 1000, 520), (1000, 200, 96)])
-def test_gated_gemm_is_silu_times_up(ops, n, inter, k):
-    """One product over the interleaved gate/up weight yields silu(x g^T) * (x u^T)."""
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+def test_gated_gemm_is_the_activated_gate_times_up(ops, n, inter, k, activation):
+    """One product over the interleaved gate/up weight yields act(x g^T) * (x u^T), in
+    every kernel that serves gated products (few tokens, 17 to 64, many)."""
     torch.manual_seed(17)
     dtype = torch.bfloat16
     x = torch.randn(n, k)
     g, u = torch.randn(inter, k) / math.sqrt(k) * 2, torch.randn(inter, k) / math.sqrt(k)
     wt = ops.interleave_gate_up(dev(g, dtype), dev(u, dtype))
     out = torch.full((n, inter), float("nan"), device="cuda", dtype=dtype)
-    ops.gemm_tiled_weight(dev(x, dtype), wt, inter, k, out, gated=True)
+    ops.gemm_tiled_weight(dev(x, dtype), wt, inter, k, out, gated=activation)
     gate = rounded(x, dtype) @ rounded(g, dtype).t()
-    want = gate * torch.sigmoid(gate) * (rounded(x, dtype) @ rounded(u, dtype).t())
+    want = gate_reference(gate, activation) * (rounded(x, dtype) @ rounded(u, dtype).t())
     close(out, want, dtype)
+    if activation == "silu":  # True stands for the activation of SwiGLU
+        again = torch.empty_like(out)
+        ops.gemm_tiled_weight(dev(x, dtype), wt, inter, k, again, gated=True)
+        assert torch.equal(again, out)
 
 
 @pytest.mark.parametrize("n, m, k", [(8, 3584, 3584), (1, 48, 4000), (33, 200, 2400), (64, 100, 2100),

@@ -378,6 +378,40 @@ def test_toy_routed_feed_forward_in_one_layer_of_two():
     assert plain.rel_err(step_whole(runner, cache, ids, [5, 1, 1, 2, 14]), want) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gated_feed_forward_with_a_gelu_gate_in_one_layer_of_two(dtype):
+    """The gate's activation is a field of the feed-forward's spec: one layer keeps
+    SiLU, the other takes GELU in its tanh form, with nothing but the spec changed."""
+    from shrike_amd.config import SwiGLUSpec
+
+    base = small_spec()
+    gelu = replace(base.blocks[1], ffn=SwiGLUSpec(intermediate_size=88, activation="gelu_tanh"))
+    spec = replace(base, blocks=(base.blocks[0], gelu))
+    w = cpu_weights(spec, seed=11)
+    if dtype == torch.bfloat16:
+        w = {k: v.to(dtype).float() for k, v in w.items()}  # the values the engine holds
+    runner, model, cache = make_runner(spec, w, dtype=dtype)
+    cfg = plain.PlainConfig(48, 88, 2, 4, 2, 16, 97, 1e-5, 1e4, False)
+    wd = {k: v.double() for k, v in w.items()}
+    ids = torch.randint(0, 97, (27,), generator=torch.Generator().manual_seed(12)).tolist()
+    n = len(ids)
+    cos, sin = plain.rope_tables(torch.arange(n), 16, 1e4)
+    x = plain.decoder_layer(cfg, wd, 0, wd["model.embed_tokens.weight"][torch.tensor(ids)], cos, sin)
+    p = "model.layers.1"
+    x = x + plain.attention_block(cfg, wd, f"{p}.self_attn", plain.rms_norm(x, wd[f"{p}.input_layernorm.weight"], 1e-5),
+                                  cos, sin, None)
+    h = plain.rms_norm(x, wd[f"{p}.post_attention_layernorm.weight"], 1e-5)
+    gate = torch.nn.functional.gelu(h @ wd[f"{p}.mlp.gate_proj.weight"].t(), approximate="tanh")
+    x = x + (gate * (h @ wd[f"{p}.mlp.up_proj.weight"].t())) @ wd[f"{p}.mlp.down_proj.weight"].t()
+    want = plain.linear(plain.rms_norm(x, wd["model.norm.weight"], 1e-5), wd["lm_head.weight"])
+    tol = 1e-5 if dtype == torch.float32 else 1.5e-2
+    assert plain.rel_err(step_whole(runner, cache, ids), want) <= tol
+    assert plain.rel_err(step_whole(runner, cache, ids, [20, 1, 1, 5]), want) <= tol
+    # and it is not the same function: the SiLU model gives other logits
+    silu_runner, _, silu_cache = make_runner(base, w, dtype=dtype)
+    assert plain.rel_err(step_whole(silu_runner, silu_cache, ids), want) > 3e-2
+
+
 # --------------------------------------------------- another position encoding
 
 
