@@ -337,6 +337,7 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
     overlap, engine.config.overlap_steps = engine.config.overlap_steps, False
     engine.step()  # takes in the step that was launched ahead, if one was, and launches none
     graphs, runner.use_graphs = runner.use_graphs, False
+    lists, runner.use_call_lists = runner.use_call_lists, False
     engine._planned = None
     try:
         for n, fn in saved.items():
@@ -354,6 +355,7 @@ def kernel_breakdown(engine, steps: int = 3) -> dict:
         for n, fn in saved.items():
             setattr(ops, n, fn)
         runner.use_graphs = graphs
+        runner.use_call_lists = lists
         engine.config.overlap_steps = overlap
         engine._planned = None
     total: dict[str, float] = {}

@@ -198,6 +198,22 @@ int shk_sample(const float* logits, int32_t* out, const float* temperature, cons
                int ld, int nucleus, void* stream);
 long long shk_sample_scratch_floats(int rows, int vocab);
 
+// A list of launches run by one call.  A shk_call names a launcher of this header that
+// takes a stream (shk_call_id gives its number by name, -1 for others) and holds its
+// arguments in order, one per slot: pointers and integers as they are, a float's bits
+// in the low 32 bits; the slot of the launcher's own stream argument is ignored and
+// `stream` is passed instead.  The calls run in order on `stream`; the first that
+// refuses its arguments ends the run with its status and message (those before it
+// have been launched).
+#define SHK_CALL_MAX_ARGS 26
+typedef struct shk_call {
+  int32_t launcher;
+  int32_t reserved;
+  int64_t args[SHK_CALL_MAX_ARGS];
+} shk_call;
+int shk_call_id(const char* name);
+int shk_run_calls(const shk_call* calls, int n, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

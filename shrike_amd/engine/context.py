@@ -47,6 +47,7 @@ class Workspace:
         # (name, dtype, shape) -> the view that was handed out last time: a step asks for
         # the same few dozen buffers layer after layer, and making a view costs a microsecond
         self._views: dict[tuple, torch.Tensor] = {}
+        self.generation = 0  # counts allocations: recorded launches name the buffers of one generation
 
     def get(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         shape = tuple(shape)
@@ -63,6 +64,7 @@ class Workspace:
                 self._outgrown.append(flat)
             flat = torch.empty(max(numel, 1), dtype=dtype, device=self.device)
             self._flat[key] = flat
+            self.generation += 1
             # views of the buffer that was replaced must not be handed out again
             self._views = {k: v for k, v in self._views.items() if k[0] != name or k[1] != dtype}
         view = flat[:numel].view(shape)
@@ -147,6 +149,8 @@ class StepContext:
     # what the parts' prepare() added: device arrays, and host-side decisions
     extras: dict = field(default_factory=dict)
     notes: dict = field(default_factory=dict)
+    # everything a step's launches may depend on, for parts that say launches_follow_shape
+    shape_key: tuple = ()
 
     def buffer(self, name: str, shape: tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         return self.workspace.get(name, shape, dtype)

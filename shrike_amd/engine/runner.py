@@ -19,12 +19,14 @@ import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, SequenceCache
+from ..kernels import lib as kernel_lib
 from ..kernels import ops
 from .context import StepContext, StepShape, Workspace
 
 GRAPH_BATCH_BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256)
 GRAPH_TABLE_QUANTUM = 64  # block-table widths of graphs are multiples of this
 MAX_GRAPHS = 24  # captured decode steps kept; the least recently used one goes first
+MAX_CALL_LISTS = 64  # recorded launch lists of other steps kept, by shape
 
 
 @dataclass
@@ -116,6 +118,14 @@ class ModelRunner:
         self._graph_workspaces: dict[int, Workspace] = {}
         self.graph_replays = 0
         self.graph_captures = 0
+        # Steps that are no graph (they hold prompt portions, or do not want every row)
+        # run their forward from a recorded list of launches when a step of the same
+        # shape has run before: one call into the library instead of one per kernel.
+        self.use_call_lists = bool(graphs) and model.launches_follow_shape()
+        self._call_lists: OrderedDict[tuple, tuple] = OrderedDict()  # shape key -> (list, logits)
+        self._call_lists_generation = -1
+        self.list_replays = 0
+        self.list_records = 0
 
     # ---------------------------------------------------------------- metadata
 
@@ -187,7 +197,9 @@ class ModelRunner:
         tables = []
         for gi in range(len(self.cache.groups)):
             need = max(1, max(len(entries[i].cache.tables[gi]) for i in order))
-            width = table_widths[gi] if table_widths else need
+            # in steps of GRAPH_TABLE_QUANTUM pages for every step: the width is part of a
+            # step's shape, and shapes that come back are run from recorded launches
+            width = table_widths[gi] if table_widths else -(-need // GRAPH_TABLE_QUANTUM) * GRAPH_TABLE_QUANTUM
             t = np.zeros((num_seqs, width), dtype=np.int64)
             for k, i in enumerate(order):
                 row = entries[i].cache.tables[gi]
@@ -233,7 +245,49 @@ class ModelRunner:
         meta = self._meta(entries, order)
         dev = self.workspace.get("step_meta", (meta.total,), torch.int32)
         self._upload(meta, dev)
-        return self._context(meta, dev, self.workspace)
+        ctx = self._context(meta, dev, self.workspace)
+        ctx.shape_key = (meta.num_tokens, meta.num_seqs, meta.num_decode, int(meta.arrays["out_rows"].size),
+                         tuple(t.shape[1] for t in meta.tables),
+                         tuple((n, int(meta.shape.extras[n].size)) for n in meta.extra_names),
+                         tuple(meta.shape.launch_key))
+        return ctx
+
+    def _forward(self, ctx: StepContext) -> torch.Tensor:
+        """The model's forward for a step that is no graph: from the recorded launches
+        of an earlier step of the same shape where there is one, else kernel by kernel
+        (and recorded).  The step's metadata is already on its way to the device; the
+        launches name the same buffers step after step, so a list stands as long as no
+        buffer of the workspace has been replaced by a larger one."""
+        if not self.use_call_lists:
+            return self.model.forward(ctx, self.layer_caches)
+        generation = self.workspace.generation
+        if self._call_lists_generation != generation:
+            self._call_lists.clear()
+            self._call_lists_generation = generation
+        key = ctx.shape_key
+        held = self._call_lists.get(key)
+        if held is not None:
+            self._call_lists.move_to_end(key)
+            calls, logits = held
+            calls.run(ops.current_stream())
+            self.list_replays += 1
+            return logits
+        kernel_lib.begin_recording()
+        try:
+            logits = self.model.forward(ctx, self.layer_caches)
+        except BaseException:
+            kernel_lib.end_recording(keep=False)
+            raise
+        calls = kernel_lib.end_recording()
+        self.list_records += 1
+        if self.workspace.generation != generation:
+            # this step grew a buffer: lists recorded before it may name the one that went
+            self._call_lists.clear()
+            self._call_lists_generation = self.workspace.generation
+        if len(self._call_lists) >= MAX_CALL_LISTS:
+            self._call_lists.popitem(last=False)
+        self._call_lists[key] = (calls, logits)
+        return logits
 
     # ------------------------------------------------------------------ graphs
 
@@ -449,7 +503,7 @@ class ModelRunner:
             logits = self._graph_step(entries, key)
         else:
             ctx = self.build_context(entries)
-            logits = self.model.forward(ctx, self.layer_caches)
+            logits = self._forward(ctx)
         for e in entries:
             e.cache.fresh_state = False
         return logits

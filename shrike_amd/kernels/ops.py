@@ -34,6 +34,11 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def current_stream() -> int:
+    """Handle of the HIP stream that launches go to now."""
+    return _stream()
+
+
 def _dev(t: torch.Tensor, name: str, dtype=None) -> int:
     if not t.is_cuda:
         raise KernelError(f"{name}: expected a device tensor (there is no CPU path)")

@@ -55,6 +55,12 @@ class DecoderModel:
                 return False
         return True
 
+    def launches_follow_shape(self) -> bool:
+        """Whether every part says that its launches follow from a step's shape and
+        launch key alone: the forward of such a model can be run again from a recorded
+        list of launches for any later step of the same shape."""
+        return all(part.launches_follow_shape for part in self.parts())
+
     def cache_specs(self) -> list:
         """Cache need of every schedule position (None for a position that
         reads another position's cache or whose mixer keeps nothing)."""

@@ -135,6 +135,12 @@ class PagedAttention(Mixer):
     reference's view (qwen.py:120-122).
     """
 
+    @property
+    def launches_follow_shape(self):
+        # the plan of a step's launches is a function of the step's shape and goes into its
+        # launch key (prepare); a position encoding of its own kind must say the same of itself
+        return self.position is None or self.position.launches_follow_shape
+
     def __init__(self, spec, width, name):
         super().__init__(spec, width, name)
         self.position = (
@@ -251,6 +257,8 @@ class PagedAttention(Mixer):
             plan.kernel = "tiles"
             seqs, q0 = portion_runs(portions, shape.num_decode, QUERY_TILE)
         plan.count = int(seqs.size)
+        # what the launches of the portions depend on beyond the step's sizes
+        shape.launch_key.append((key, plan.kernel, plan.small, plan.portion_splits, plan.first_token, plan.count))
         tag = f"{h}:{hkv}:{d}:{s.window or 0}"
         plan.seq_name, plan.q0_name = f"attention_seq:{tag}", f"attention_q0:{tag}"
         shape.add(plan.seq_name, seqs)

@@ -119,6 +119,13 @@ class Part:
     # device data on the host, or launches work whose shape depends on the data);
     # a model with such a part runs every step kernel by kernel.
     graph_safe = True
+    # True for a part whose launches (kernels, their scalar arguments, the buffers
+    # they name) follow from the step's shape alone: the numbers of tokens, sequences,
+    # single tokens and wanted rows, the widths of the block tables, the sizes of the
+    # arrays that parts added, and the step's launch key.  Steps of equal shape then
+    # run such a model's forward from a recorded list of launches.  A part that
+    # decides anything else on the host per step must put it into the launch key.
+    launches_follow_shape = False
 
     def __init__(self, spec, width: int, name: str):
         self.spec = spec

@@ -28,6 +28,10 @@ class PreNormResidualBlock(Block):
     def graph_safe(self):
         return all(part.graph_safe for part in self.parts)
 
+    @property
+    def launches_follow_shape(self):
+        return all(part.launches_follow_shape for part in self.parts)
+
     def load(self, tensors, runtime):
         for part in self.parts:
             part.load(tensors, runtime)

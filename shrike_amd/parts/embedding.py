@@ -12,6 +12,8 @@ class TokenEmbedding(Embedding):
     """x[n] = table[token_ids[n]], widened to float32, without any scaling
     (reference: shrike/models/qwen.py:156,161)."""
 
+    launches_follow_shape = True
+
     def params(self):
         return [ParamSpec(f"{self.name}.weight", (self.spec.vocab_size, self.width), init="embedding")]
 

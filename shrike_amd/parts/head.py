@@ -13,6 +13,8 @@ class LinearHead(Head):
     file carries no output matrix, W is the embedding table itself
     (qwen.py:211-212)."""
 
+    launches_follow_shape = True
+
     def __init__(self, spec, width, name):
         super().__init__(spec, width, name)
         self.tied_to = None

@@ -13,6 +13,8 @@ class SwiGLU(FeedForward):
     are joined into one weight at load time, so that one product yields the
     activated values."""
 
+    launches_follow_shape = True
+
     def params(self):
         inter, h = self.spec.intermediate_size, self.width
         return [

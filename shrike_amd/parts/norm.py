@@ -12,6 +12,8 @@ class RMSNorm(Norm):
     """y = x * rsqrt(mean(x^2) + eps) * weight in float32, one cast at the end
     (reference: shrike/models/qwen.py:70-74)."""
 
+    launches_follow_shape = True
+
     def params(self):
         return [ParamSpec(f"{self.name}.weight", (self.width,), init="norm", keep_float32=True)]
 

@@ -13,6 +13,8 @@ class RotaryHalf(PositionEncoding):
     float32(p) * inv_freq[i] (:86).  The rotation itself runs inside the
     cache-write kernel."""
 
+    launches_follow_shape = True
+
     def load(self, tensors, runtime):
         d = int(self.spec.rotary_dim)
         inv_freq = 1.0 / (float(self.spec.theta) ** (torch.arange(0, d, 2).float() / d))

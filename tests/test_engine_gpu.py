@@ -556,3 +556,67 @@ def test_command_line_builds_a_random_model_from_a_config(tmp_path, capsys):
         runs.append([int(t) for t in capsys.readouterr().out.split()])
     assert len(runs[0]) == 6 and runs[0] == runs[1]
     assert main(["--random-config", str(tmp_path / "absent.json"), "--prompt-len", "3"]) == 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_recorded_launch_lists_equal_kernel_by_kernel_steps(dtype, model_root):
+    """Steps that are no graph (prompt portions beside single tokens, rows that are not
+    wanted) run from the recorded launches of an earlier step of the same shape.  With
+    shapes that come back, shapes that do not, and a step in between that outgrows the
+    buffers (which drops every list), the logits are bit for bit those of a runner that
+    launches every kernel from Python."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner, StepEntry
+
+    model_dir = make_model_dir("D", model_root, dtype=dtype, mode="unit")
+    model, rt, cfg = load_model(model_dir, dtype)
+    assert model.launches_follow_shape()
+    rng = random.Random(3)
+    ids = [[rng.randrange(cfg.vocab_size) for _ in range(400)] for _ in range(3)]
+    # (portion of sequence 0, portion of sequence 1, single token of sequence 2?) per step: the same
+    # shapes several times over, at other positions, then a larger step, then the first shapes again
+    plan = ([(24, 0, True)] * 4 + [(24, 9, True)] * 3 + [(7, 0, False)] * 2 + [(120, 40, True)] + [(24, 0, True)] * 2
+            + [(24, 9, True)] * 2)
+
+    def run(graphs):
+        cache = CacheManager(model.cache_specs(), 16, 90, enable_prefix_caching=False)
+        cache.allocate(rt.dtype, rt.device)
+        runner = ModelRunner(model, cache, rt, graphs=graphs)
+        seqs = [cache.new_sequence() for _ in ids]
+        at = [0, 0, 0]
+        outs = []
+        for n0, n1, single in plan:
+            entries = []
+            for s, n in ((0, n0), (1, n1), (2, 1 if single else 0)):
+                if n:
+                    cache.append(seqs[s], at[s], n)
+                    want = [n - 1] if s != 1 else [0, n // 2]
+                    entries.append(StepEntry(seqs[s], ids[s][at[s] : at[s] + n], at[s], want))
+                    at[s] += n
+            outs.append(runner.step(entries).cpu().clone())
+            for s in range(3):
+                cache.trim(seqs[s], at[s])
+        return outs, runner
+
+    plain_outs, plain_runner = run(False)
+    listed_outs, listed_runner = run(True)
+    assert plain_runner.list_replays == 0 and plain_runner.list_records == 0
+    # shapes (24, 0), (24, 9), (7, 0), (120, 40), and (24, 0), (24, 9) once more after the large step
+    assert listed_runner.list_records == 6 and listed_runner.list_replays == len(plan) - 6
+    for a, b in zip(plain_outs, listed_outs):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
+
+
+def test_a_model_with_a_part_that_decides_on_the_host_is_never_run_from_a_list(model_root):
+    """Only parts that say their launches follow from the step's shape are recorded."""
+    from shrike_amd.cache import CacheManager
+    from shrike_amd.engine.loading import load_model
+    from shrike_amd.engine.runner import ModelRunner
+
+    model, rt, _ = load_model(make_model_dir("A", model_root), "float32")
+    cache = CacheManager(model.cache_specs(), 4, 8, enable_prefix_caching=False)
+    assert ModelRunner(model, cache, rt).use_call_lists
+    model.blocks[0].ffn.launches_follow_shape = False  # as a part of the user's own would have it
+    assert not model.launches_follow_shape()
+    assert not ModelRunner(model, cache, rt).use_call_lists
