@@ -1,7 +1,7 @@
 """Configurations at the edges of what the kernels take: a width that is no
 multiple of 8, heads * head_dim != hidden, 32 query heads on one key/value
-head, head sizes 16, 80 and 256, vocabularies that are no power of two, tied
-weights; each in float32 and bfloat16, with pages of 16 (MFMA attention where
+head, 16 and 17 on one, head sizes 16, 80, 96, 160 and 256, a window, vocabularies
+that are no power of two, tied weights; each in float32 and bfloat16, with pages of 16 (MFMA attention where
 the shape allows) and of 4 (general kernel)."""
 
 import tempfile
@@ -26,6 +26,17 @@ CASES = {
                          num_key_value_heads=2, head_dim=256, vocab_size=999, tie_word_embeddings=True),
     "width130_group3": dict(hidden_size=130, intermediate_size=70, num_hidden_layers=1,
                             num_attention_heads=9, num_key_value_heads=3, head_dim=64, vocab_size=513),
+    # 16 query heads on a key/value head is the most the matrix-instruction kernels take; a
+    # head size above 128 leaves prompt portions to the kernel that works tile by tile
+    "head160_group16": dict(hidden_size=88, intermediate_size=120, num_hidden_layers=2,
+                            num_attention_heads=16, num_key_value_heads=1, head_dim=160, vocab_size=4099),
+    # one head more than that: the general kernel serves it
+    "group17": dict(hidden_size=68, intermediate_size=80, num_hidden_layers=1, num_attention_heads=17,
+                    num_key_value_heads=1, head_dim=32, vocab_size=211),
+    # seven heads per group of 96 with a window from the second layer on
+    "head96_group7_window": dict(hidden_size=120, intermediate_size=200, num_hidden_layers=3,
+                                 num_attention_heads=14, num_key_value_heads=2, head_dim=96, vocab_size=8200,
+                                 use_sliding_window=True, sliding_window=33, max_window_layers=1),
 }
 
 
@@ -53,6 +64,7 @@ def test_odd_shapes(name):
                     cache.append(seq, p, n)
                     outs.append(runner.step([StepEntry(seq, ids[p : p + n], p, list(range(n)))]).cpu().clone())
                     p += n
+                    cache.trim(seq, p)
                 err = rel_err(torch.cat(outs), want)
                 assert err <= tol, f"{name} {dtype} page {page_size}: rel err {err:.2e}"
                 cache.free(seq)
