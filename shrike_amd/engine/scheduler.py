@@ -29,6 +29,22 @@ from ..cache.manager import CacheManager
 from .request import Request, Status
 
 
+class _StepPlan:
+    """What one schedule() call has handed out so far, and what is left of the budget."""
+
+    def __init__(self, budget: int):
+        self.budget = budget
+        self.singles: list[tuple[Request, int]] = []
+        self.portions: list[tuple[Request, int]] = []
+
+    def take(self, req: Request, n: int) -> None:
+        (self.singles if n == 1 else self.portions).append((req, n))
+        self.budget -= n
+
+    def batch(self) -> list[tuple[Request, int]]:
+        return self.singles + self.portions
+
+
 class Scheduler:
     def __init__(self, cache: CacheManager, max_tokens_per_step: int = 512, max_running: int = 256):
         self.cache = cache
@@ -63,53 +79,49 @@ class Scheduler:
         return newest
 
     def schedule(self) -> list[tuple[Request, int]]:
-        singles: list[tuple[Request, int]] = []
-        portions: list[tuple[Request, int]] = []
-        budget = self.max_tokens_per_step
+        """The next step's (request, number of its next tokens), requests with one
+        token first (the step function's order), each group in admission order."""
+        step = _StepPlan(self.max_tokens_per_step)
+        self._serve_running(step)
+        self._admit_waiting(step)
+        return step.batch()
 
-        for req in list(self.running):
-            if budget == 0:
-                break
-            if req.status is not Status.RUNNING:  # preempted earlier in this step
-                continue
-            n_new = min(req.num_tokens - req.num_computed_tokens, budget)
-            if n_new <= 0:
-                continue
-            while n_new and not self.cache.can_append(req.cache, req.num_computed_tokens, n_new):
+    def _serve_running(self, step: "_StepPlan") -> None:
+        """Rule 1 and 3: every running request gets its next tokens while the budget
+        lasts; the pages for them are taken from the newest running requests if
+        need be."""
+        for req in tuple(self.running):
+            if step.budget == 0:
+                return
+            if req.status is not Status.RUNNING:
+                continue  # preempted for an older request a moment ago
+            wanted = min(req.num_tokens - req.num_computed_tokens, step.budget)
+            while wanted > 0 and not self.cache.can_append(req.cache, req.num_computed_tokens, wanted):
                 if self._preempt_newest() is req:
-                    n_new = 0  # it was the newest itself: it sits this step out
-            if n_new == 0:
-                continue
-            self.cache.append(req.cache, req.num_computed_tokens, n_new)
-            (singles if n_new == 1 else portions).append((req, n_new))
-            budget -= n_new
+                    wanted = 0  # it was the newest itself: it sits this step out
+            if wanted > 0:
+                self.cache.append(req.cache, req.num_computed_tokens, wanted)
+                step.take(req, wanted)
 
-        while (
-            self.waiting
-            and budget > 0
-            and len(self.running) < self.max_running
-            and self.cache.slots.num_free > 0
-        ):
+    def _admit_waiting(self, step: "_StepPlan") -> None:
+        """Rule 2: the head of the waiting queue, again and again, while budget, running
+        places, state slots and pages allow; nothing overtakes a head that does not fit."""
+        while self.waiting and step.budget > 0 and len(self.running) < self.max_running \
+                and self.cache.slots.num_free > 0:
             req = self.waiting[0]
             seq = self.cache.new_sequence()
-            # A resumed request recomputes what it generated before it was preempted too.
-            known = req.num_tokens
+            # a request that was preempted recomputes what it had generated as well
             cached = self.cache.match_prefix(seq, req.token_ids[: req.num_prompt_tokens])
-            n_new = min(known - cached, budget)
-            if not self.cache.can_append(seq, cached, n_new):
-                self.cache.free(seq)  # also drops the references a prefix match took
-                break
+            wanted = min(req.num_tokens - cached, step.budget)
+            if not self.cache.can_append(seq, cached, wanted):
+                self.cache.free(seq)  # the slot, and the references that the prefix match took
+                return
+            self.cache.append(seq, cached, wanted)
             self.waiting.popleft()
-            req.cache = seq
-            req.num_computed_tokens = cached
+            req.cache, req.num_computed_tokens, req.status = seq, cached, Status.RUNNING
             req.hashed_pages, req.last_hash = 0, None
-            self.cache.append(seq, cached, n_new)
-            req.status = Status.RUNNING
             self.running.append(req)
-            (singles if n_new == 1 else portions).append((req, n_new))
-            budget -= n_new
-
-        return singles + portions
+            step.take(req, wanted)
 
     def plan_decode_step(self) -> list[tuple[Request, int]] | None:
         """What the next schedule() will return if every running request goes on
