@@ -405,6 +405,71 @@ def run_mixed(engine, cfg, decodes: int, budget: int, seed: int) -> dict:
             "tokens_per_s": round(budget / mean * 1e3, 1)}
 
 
+def run_products(cfg, tokens: list[int]) -> dict:
+    """Microseconds of each of a layer's four products (and of the output head) with
+    the engine's kernels and, beside them, with the vendor library's matrix product
+    (torch.matmul) on the same sizes: a yardstick only, the engine never calls it.
+    The engine's gate/up product includes the gate's activation and writes half the
+    columns; its products of few tokens include no reader of their shares of k."""
+    import statistics
+
+    import torch
+
+    from shrike_amd.kernels import ops
+
+    dev = "cuda:0"
+
+    def graph_us(fn, repeats=5):
+        fn()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(repeats):
+                fn()
+        times = []
+        for _ in range(5):
+            torch.cuda.synchronize()
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            graph.replay()
+            b.record()
+            torch.cuda.synchronize()
+            times.append(a.elapsed_time(b) * 1e3 / repeats)
+        return statistics.median(times)
+
+    h, inter = cfg.hidden_size, cfg.intermediate_size
+    qkv = (cfg.num_attention_heads + 2 * cfg.num_key_value_heads) * cfg.head_dim
+    shapes = [("qkv", qkv, h, False), ("o", h, cfg.num_attention_heads * cfg.head_dim, False),
+              ("gate_up", inter, h, True), ("down", h, inter, False), ("lm_head", cfg.vocab_size, h, False)]
+    out = {}
+    for n in tokens:
+        for name, m, k, gated in shapes:
+            if name == "lm_head" and n > 64:
+                continue  # the head only ever sees the rows whose logits are wanted
+            rows = 2 * m if gated else m
+            w = (torch.randn(rows, k, device=dev) * k**-0.5).to(torch.bfloat16)
+            x = torch.randn(n, k, device=dev).to(torch.bfloat16)
+            y = torch.empty(n, rows, device=dev, dtype=torch.bfloat16)
+            library = graph_us(lambda: torch.matmul(x, w.t(), out=y))
+            if gated:
+                tiled = ops.interleave_gate_up(w[:m].contiguous(), w[m:].contiguous())
+            else:
+                tiled = ops.retile_weight(w)
+            del w
+            splits = 1 if gated else ops.gemm_splits(n, m, k)
+            z = (torch.empty(splits, n, m, device=dev) if splits > 1
+                 else torch.empty(n, m, device=dev, dtype=torch.bfloat16))
+            if gated:
+                own = graph_us(lambda: ops.gemm_tiled_weight(x, tiled, m, k, z, gated="silu"))
+            else:
+                own = graph_us(lambda: ops.gemm_tiled_weight(x, tiled, m, k, z, splits=splits))
+            out[f"{name}_n{n}"] = {"own_us": round(own, 1), "library_us": round(library, 1), "k_shares": splits}
+            print(f"[bench] {n:5d} tokens {name:8s} {rows:6d} x {k:5d}: own {own:7.1f} us ({splits} shares of k), "
+                  f"library {library:7.1f} us", file=sys.stderr)
+            del tiled, x, y, z
+    return out
+
+
 def main() -> int:
     global CONTEXT_END
     started = time.perf_counter()
@@ -434,6 +499,9 @@ def main() -> int:
     ap.add_argument("--offline", type=int, default=0, metavar="REQUESTS",
                     help="instead: the reference's offline throughput run, REQUESTS short prompts with 32 to "
                          "256 new tokens each through generate() (prints its own JSON line)")
+    ap.add_argument("--products", action="store_true",
+                    help="instead: time a layer's matrix products at 1 to 2,048 tokens with the engine's kernels "
+                         "and, as a yardstick, with the vendor library (prints its own JSON line)")
     ap.add_argument("--seed", type=int, default=0)
     args = ap.parse_args()
     if args.gpus != 1:
@@ -462,6 +530,13 @@ def main() -> int:
         raw["num_hidden_layers"] = args.layers
     cfg = Qwen2Config.from_dict(raw)
     spec = build_spec(cfg)
+    if args.products:
+        products = run_products(cfg, [1, 8, 64, 512, PROMPT_LEN])
+        print(json.dumps({
+            "metric": f"us of a layer's matrix products, own kernels and vendor library (Qwen2.5-{args.shape.upper()} shape)",
+            "unit": "us", "n_gpus": 1, "higher_is_better": False, "dtype": "bf16",
+            "data": "synthetic: random operands", "products": products}))
+        return 0
     if args.offline:
         offline = run_offline(cfg, spec, args.offline, args.seed)
         print(json.dumps({
