@@ -55,6 +55,30 @@ __device__ __forceinline__ float row16_sum(float v) {
   return v;
 }
 
+// Maximum and sum over the four lanes j, j + 16, j + 32, j + 48 (one query's scores in
+// the transposed products), in every one of them.  Two swaps of the vector unit (gfx950's
+// v_permlane16_swap / v_permlane32_swap) instead of two trips through the LDS crossbar,
+// which the chunk's chain of dependent steps would wait for: with rows of 16 lanes r0 r1
+// r2 r3, the first swap of v with itself gives (r0 r0 r2 r2) and (r1 r1 r3 r3), the
+// second, of what they combine to, (a a a a) and (b b b b).  Everything here is written
+// so that the compiler sees it: an instruction in asm would hide from it what the
+// swaps' operands have to wait for.
+__device__ __forceinline__ float bits_as_float(unsigned v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ float lanes4_max(float v) {
+  const unsigned b = __builtin_bit_cast(unsigned, v);
+  const auto rows = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  const unsigned h = __builtin_bit_cast(unsigned, fmaxf(bits_as_float(rows[0]), bits_as_float(rows[1])));
+  const auto halves = __builtin_amdgcn_permlane32_swap(h, h, false, false);
+  return fmaxf(bits_as_float(halves[0]), bits_as_float(halves[1]));
+}
+__device__ __forceinline__ float lanes4_sum(float v) {
+  const unsigned b = __builtin_bit_cast(unsigned, v);
+  const auto rows = __builtin_amdgcn_permlane16_swap(b, b, false, false);
+  const unsigned h = __builtin_bit_cast(unsigned, bits_as_float(rows[0]) + bits_as_float(rows[1]));
+  const auto halves = __builtin_amdgcn_permlane32_swap(h, h, false, false);
+  return bits_as_float(halves[0]) + bits_as_float(halves[1]);
+}
+
 constexpr int kPStride = 40;  // bf16 elements per row of the P tile in LDS (32 + padding)
 
 // A window of 64 entries of a sequence's block table held across the lanes of
@@ -431,8 +455,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
           if (g0 + e > pos || g0 + e < lo) sc[e] = -INFINITY;
       }
       float mx = max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), fmaxf(sc[6], sc[7]));
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = lanes4_max(mx);
       const float m_new = fmaxf(m, mx);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m - m_safe);
@@ -502,8 +525,7 @@ __global__ void __launch_bounds__(kDecodeWaves* kWave)
         attend(buf[u], kb);
       }
     }
-    l += __shfl_xor(l, 16, kWave);
-    l += __shfl_xor(l, 32, kWave);
+    l = lanes4_sum(l);
   }
 
   // ---- the wavefronts' results become one: common maximum, sums in wavefront order
@@ -887,8 +909,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
           if (g0 + e > q_pos[u] || g0 + e < q_lo[u]) sc[e] = -INFINITY;
       }
       float mx = max3(max3(sc[0], sc[1], sc[2]), max3(sc[3], sc[4], sc[5]), fmaxf(sc[6], sc[7]));
-      mx = fmaxf(mx, __shfl_xor(mx, 16, kWave));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, kWave));
+      mx = lanes4_max(mx);
       const float m_new = fmaxf(m[u], mx);
       const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
       const float alpha = __builtin_amdgcn_exp2f(m[u] - m_safe);
@@ -946,8 +967,7 @@ __global__ void __launch_bounds__(WAVES* kWave) __attribute__((amdgpu_waves_per_
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     float total = l[u];
-    total += __shfl_xor(total, 16, kWave);
-    total += __shfl_xor(total, 32, kWave);
+    total = lanes4_sum(total);
     if (j >= unit_rows[u]) continue;
     if (nsplit > 1) {
       // a share's result, for attention_merge_kernel: O [row][share][D], then (maximum,

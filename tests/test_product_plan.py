@@ -157,3 +157,4 @@ def test_where_a_product_runs_in_two_parts():
     assert ops.gemm_parts(512, 18944, 3584, True) == 2    # 296 tiles of 256 x 256: 256 + 40
     assert ops.gemm_parts(2048, 18944, 3584, True) == 1   # 1,184 tiles: the rest would take a round of its own anyway
     assert ops.gemm_parts(512, 3584, 18944) == 1          # shares of k instead
+    assert ops.gemm_parts(2048, 13824, 5120, True) == 2   # 864 tiles: three whole rounds, then 96 tiles' rows in smaller tiles
