@@ -29,3 +29,14 @@ def test_offline_run_and_decode_run_on_a_tiny_model():
     assert run["context_end"] - run["context_start"] == 10 and run["tok_s"] > 0
     sampled = bench.run_decode(engine, cfg, 4, steps=10, warmup=2, seed=6, prompt_len=40, temperature=0.8, top_p=0.9)
     assert sampled["context_end"] - sampled["context_start"] == 10
+
+
+def test_products_mode_times_every_product_of_a_layer_both_ways():
+    import shrike_amd.models  # noqa: F401
+    from shrike_amd.models.qwen2 import Qwen2Config
+
+    cfg = Qwen2Config.from_dict(dict(CONFIGS["D"], torch_dtype="bfloat16"))
+    got = bench.run_products(cfg, [8, 200])
+    assert set(got) == {f"{name}_n{n}" for n in (8, 200) for name in ("qkv", "o", "gate_up", "down")} | {"lm_head_n8"}
+    for entry in got.values():
+        assert entry["own_us"] > 0 and entry["library_us"] > 0 and entry["k_shares"] >= 1
