@@ -175,9 +175,9 @@ def run_decode(engine, cfg, batch: int, steps: int, warmup: int, seed: int,
     }
 
 
-def run_chunked_prefill(engine, cfg, seed: int, budget: int = 512) -> float:
-    """Milliseconds until a PROMPT_LEN-token prompt has its first token when the
-    scheduler cuts it into portions of `budget` tokens (the reference's default)."""
+def run_chunked_prefill(engine, cfg, seed: int, budget: int = 512, prompt_len: int = PROMPT_LEN) -> float:
+    """Milliseconds until a prompt of `prompt_len` tokens has its first token when the
+    scheduler cuts it into portions of `budget` tokens (the reference's default: 512)."""
     import torch
 
     from shrike_amd import SamplingParams
@@ -187,7 +187,7 @@ def run_chunked_prefill(engine, cfg, seed: int, budget: int = 512) -> float:
     best = None
     try:
         for _ in range(2):
-            engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(PROMPT_LEN)],
+            engine.add_request([rng.randrange(cfg.vocab_size) for _ in range(prompt_len)],
                                SamplingParams(max_new_tokens=1, ignore_eos=True))
             torch.cuda.synchronize()
             t0 = time.perf_counter()
@@ -197,7 +197,7 @@ def run_chunked_prefill(engine, cfg, seed: int, budget: int = 512) -> float:
                 steps += 1
             torch.cuda.synchronize()
             dt = time.perf_counter() - t0
-            assert steps == -(-PROMPT_LEN // budget)
+            assert steps == -(-prompt_len // budget)
             best = dt if best is None else min(best, dt)
     finally:
         engine.scheduler.max_tokens_per_step = saved
@@ -595,6 +595,11 @@ def main() -> int:
         print(f"[bench] 2,048-token prompt in portions of 512: {more_points['prefill_2048_budget512_ms']} ms",
               file=sys.stderr)
         if 8 * (16000 // PAGE_SIZE + 16) <= engine.cache.num_pages:
+            long_ms = run_chunked_prefill(engine, cfg, args.seed, budget=PROMPT_LEN, prompt_len=16000)
+            more_points["prefill_16000_budget2048_ms"] = round(long_ms, 2)
+            more_points["prefill_16000_bf16_frac"] = round(
+                prefill_flops(cfg, 16000) / (long_ms * 1e-3) / BF16_PEAK_FLOPS, 4)
+            print(f"[bench] 16,000-token prompt in portions of {PROMPT_LEN}: {long_ms:.1f} ms", file=sys.stderr)
             long_run = run_decode(engine, cfg, 8, min(args.steps, 40), args.warmup, args.seed + 300, 16000)
             more_points["decode_b8_ctx16000"] = round(long_run["tok_s"], 1)
             more_points["decode_b8_ctx16000_hbm_frac"] = round(long_run["gb_s"] / HBM_PEAK_GBS, 4)
