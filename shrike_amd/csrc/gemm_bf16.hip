@@ -1331,6 +1331,27 @@ extern "C" int shk_gemm_bf16_splits(int n, int m, int k) {
   if (n <= 16) {
     split = 8192 / (mblocks * 4), most = ktiles / 16;
     if (split > 16) split = 16;
+    // A matrix of less than 96 MiB is read sooner than its kernel starts and ends: what
+    // counts is how long the busiest compute unit's workgroups walk and what every share
+    // costs by itself and in the kernel that adds the shares up.  Workgroups on one compute
+    // unit take turns at its intake, so a launch takes about (workgroups per compute unit,
+    // rounded up) x (k-tiles per share) x 0.057 us, and a share about 0.45 us.  Measured
+    // with 8 tokens, product + reading norm: 3584 x 3584 in 2 shares 10.1 us, in 3 11.4,
+    // in 4 11.0, in 7 11.8 (224, 336, 448, 784 workgroups on 256 compute units); 4608 x
+    // 3584 in 2 13.8, in 3 12.4, in 4 13.6, in 7 12.9; 5120 x 5120 in 3 14.9, in 6 16.4;
+    // 7168 x 5120 whole 17.6, in 4 19.5.
+    if (static_cast<long long>(mblocks) * ktiles <= 96 * 1024) {
+      const int groups = mblocks >= 128 ? (mblocks + 1) / 2 : mblocks;  // (pairs of row blocks)
+      const int top = most < 1 ? 1 : (most > 16 ? 16 : most);
+      int best = 1;
+      double least = 0.0;
+      for (int shares = 1; shares <= top; ++shares) {
+        const int turns = (groups * shares + kDies * kDieUnits - 1) / (kDies * kDieUnits);
+        const double us = turns * ((ktiles + shares - 1) / shares) * 0.057 + shares * 0.45;
+        if (shares == 1 || us < least) least = us, best = shares;
+      }
+      return best;
+    }
   } else {
     split = 2048 / mblocks, most = ktiles / 28;
     if (split > 8) split = 8;

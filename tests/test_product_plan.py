@@ -34,6 +34,17 @@ def test_matrices_that_fill_the_chip_are_not_split():
     assert ops.gemm_splits(512, 5120, 13824) > 1      # 80 tiles of 256 x 128
 
 
+def test_small_matrices_of_a_decode_step_take_few_shares():
+    """Up to 16 tokens, a matrix below 96 MiB: the count of shares that keeps the busiest
+    compute unit's workgroups shortest, each share costing something by itself."""
+    assert ops.gemm_splits(8, 3584, 3584) == 2    # 112 pairs of row blocks: 224 workgroups, one each
+    assert ops.gemm_splits(8, 4608, 3584) == 3    # 144 pairs: 2 shares would give 32 compute units two each
+    assert ops.gemm_splits(8, 5120, 5120) == 3
+    assert ops.gemm_splits(8, 7168, 5120) == 1    # 224 pairs fill the chip unsplit
+    assert ops.gemm_splits(8, 3584, 18944) == 9   # 130 MiB: a matter of bandwidth, many workgroups
+    assert ops.gemm_splits(8, 896, 896) == 1      # 28 k-tiles: too few to share
+
+
 def test_key_splits_of_decode_attention_depend_on_the_buckets_only():
     """A graph is captured for a bucket of sequences and of context; every step
     that it replays must split the keys as the captured one did."""
