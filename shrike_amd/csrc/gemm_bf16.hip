@@ -1244,8 +1244,11 @@ static void launch_big(hipStream_t s, const bf16* ap, int lda, int n, int k, con
 // (TFLOP/s per compute unit: 4.75, 4.0, and for the smallest tile 3.0 with the
 // compute unit to itself or 1.5 for each of two), plus what a kernel costs
 // anyway, plus writing and reading the float32 parts of a split product at
-// 4 TB/s.  It reproduces the measured times of the 7B and 14B matrices at 512
-// tokens within 10 %.
+// 3 TB/s (at 4 TB/s the estimate took shares that lost with their reader: the
+// 14B down matrix at 4,096 tokens 701 us in two shares against 553 whole, the 14B
+// QKV matrix at 768 tokens 100 us in three against 87, the 7B QKV matrix at 512
+// tokens 54 in three against 51).  It reproduces the measured times of the 7B
+// and 14B matrices at 512 tokens within 10 %.
 static double big_estimate(int shape, int split, int n, int wblocks, int m, int k) {
   const int rows = shape == 2 ? 128 : 256, tokens = shape == 0 ? 256 : 128;
   const long long tiles =
@@ -1263,7 +1266,7 @@ static double big_estimate(int shape, int split, int n, int wblocks, int m, int 
   double us = rounds * 2.0 * rows * tokens * share / (rate * 1e6) + 5.0;
   // (tokens counted in whole tiles of 128: the choice is then the same for every
   // number of tokens that a captured decode step of 128 or 256 rows may stand for)
-  if (split > 1) us += 2.0 * split * ((n + 127) / 128 * 128.0) * m * 4.0 / 4e6;
+  if (split > 1) us += 2.0 * split * ((n + 127) / 128 * 128.0) * m * 4.0 / 3e6;
   return us;
 }
 
